@@ -1,0 +1,173 @@
+/*
+ * pink_hip.h -- C ABI of the MI355X (gfx950) implementation of PINK's GPU
+ * training and mapping step.
+ *
+ * One context replaces the device half of one reference
+ *   pink::Trainer<SOMLayout, DataLayout, float, true>   (src/SelfOrganizingMapLib/Trainer.h:201-335)
+ * or
+ *   pink::Mapper <SOMLayout, DataLayout, float, true>   (src/SelfOrganizingMapLib/Mapper.h:129-230)
+ * i.e. everything those classes reach in src/CudaLib: the spatial transformer
+ * (CudaLib/generate_rotated_images.h:57-294), the distance matrix + argmin
+ * (CudaLib/generate_euclidean_distance_matrix.h:26-270) and the BMU search +
+ * neuron update (CudaLib/update_neurons.h:55-85).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; all `host_*` pointers are host memory, all
+ *     `dev_*` pointers are device memory of the context's device;
+ *   - every function returns PINK_HIP_OK (0) or a negative pink_hip_status and never
+ *     terminates the process (the reference's gpuErrchk calls exit(),
+ *     CudaLib/CudaLib.h:20-29); pink_hip_last_error() gives the message the C++
+ *     caller turns into pink::exception;
+ *   - a context owns one HIP stream and all its device buffers, shares no global
+ *     state with other contexts, and must not be used from two threads at once;
+ *   - results follow the reference CPU path: rotated pixels and trained weights
+ *     bit-for-bit, float32 distances in the CPU's summation order, integer
+ *     (uint8/uint16) distances as exact integer sums of squared differences of
+ *     q = T(x * (2^bits - 1)) (CudaLib/copy_and_transform_kernel.h:27-28), lowest
+ *     index on ties everywhere.
+ */
+#ifndef PINK_HIP_H
+#define PINK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PINK_HIP_ABI_VERSION 1
+
+typedef enum pink_hip_status {
+    PINK_HIP_OK = 0,
+    PINK_HIP_EINVAL = -1,   /* bad argument; message as the reference's pink::exception */
+    PINK_HIP_ENOMEM = -2,   /* host or device allocation failed                         */
+    PINK_HIP_EDEVICE = -3,  /* a HIP call failed; message holds hipGetErrorString       */
+    PINK_HIP_ESTATE = -4    /* call not valid for this context (e.g. train on a mapper) */
+} pink_hip_status;
+
+/* src/UtilitiesLib/DataType.h:16-21 */
+typedef enum { PINK_HIP_FLOAT = 0, PINK_HIP_UINT16 = 1, PINK_HIP_UINT8 = 2 } pink_hip_data_type;
+/* src/UtilitiesLib/EuclideanDistanceShape.h:14-18 */
+typedef enum { PINK_HIP_QUADRATIC = 0, PINK_HIP_CIRCULAR = 1 } pink_hip_ed_shape;
+/* src/UtilitiesLib/Interpolation.h:15-19 */
+typedef enum { PINK_HIP_NEAREST_NEIGHBOR = 0, PINK_HIP_BILINEAR = 1 } pink_hip_interpolation;
+
+/* src/UtilitiesLib/Layout.h:13-17 */
+typedef enum { PINK_HIP_CARTESIAN = 0, PINK_HIP_HEXAGONAL = 1 } pink_hip_som_layout;
+/* src/UtilitiesLib/DistributionFunctor.h: StepFunctor, GaussianFunctor, UnityGaussianFunctor, MexicanHatFunctor */
+typedef enum { PINK_HIP_STEP = 0, PINK_HIP_GAUSSIAN = 1, PINK_HIP_UNITY_GAUSSIAN = 2, PINK_HIP_MEXICAN_HAT = 3 } pink_hip_functor;
+
+/* Which distance kernel a context uses (debugging / measurement knob). */
+typedef enum {
+    PINK_HIP_KERNEL_AUTO = 0,   /* float32: sequential-FMA VALU kernel; integer modes: int8 MFMA */
+    PINK_HIP_KERNEL_VALU = 1,   /* integer modes on the vector ALU in exact int32/int64          */
+    PINK_HIP_KERNEL_MFMA = 2
+} pink_hip_kernel_choice;
+
+/*
+ * The constructor arguments of Trainer<...,true> (Trainer.h:211-215) and
+ * Mapper<...,true> (Mapper.h:134-137), flattened.  The SOM layout itself does not
+ * reach the device: it only shapes `update_factors`, the N x N matrix
+ * TrainerCommon precomputes (Trainer.h:62,69-76).
+ */
+typedef struct pink_hip_config {
+    uint32_t som_size;        /* N  = som_layout.size()                                  */
+    uint32_t channels;        /* C  = 1 for CartesianLayout<2> data, depth for <3>       */
+    uint32_t image_dim;       /* I  : images are C x I x I, row-major, channel first     */
+    uint32_t neuron_dim;      /* D  : neurons are C x D x D                              */
+    uint32_t num_rot;         /* number_of_rotations: 1 or a multiple of 4               */
+    uint32_t use_flip;        /* 0 / 1                                                   */
+    uint32_t interpolation;   /* pink_hip_interpolation                                  */
+    uint32_t ed_dim;          /* euclidean_distance_dim                                  */
+    uint32_t ed_shape;        /* pink_hip_ed_shape                                       */
+    uint32_t ed_type;         /* pink_hip_data_type (euclidean_distance_type)            */
+    const float *update_factors; /* host, N*N floats, row = BMU; NULL makes a mapper     */
+    int32_t  device;          /* HIP device ordinal                                      */
+    uint32_t max_batch;       /* images per launch group when mapping; 0 = choose        */
+    uint32_t kernel_choice;   /* pink_hip_kernel_choice                                  */
+} pink_hip_config;
+
+typedef struct pink_hip_ctx pink_hip_ctx;
+
+/* Replaces the constructors Trainer.h:211-260 / Mapper.h:134-179 (device allocation,
+ * cos/sin tables, circle tables, upload of the update factors).  Argument errors the
+ * reference throws (Trainer.h:66-67, Mapper.h:59-66, CudaLib/generate_rotated_images.h:51,120)
+ * are reported here with the same text. */
+int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg);
+void pink_hip_destroy(pink_hip_ctx *ctx);
+
+/* Message of the last failing call on `ctx` (or of the last failing
+ * pink_hip_create on this thread when ctx is NULL).  Never NULL. */
+const char *pink_hip_last_error(const pink_hip_ctx *ctx);
+
+/* Upload the SOM (N * C*D*D floats): the `d_som(som.get_data())` initialisers at
+ * Trainer.h:218 and Mapper.h:140. */
+int pink_hip_set_som(pink_hip_ctx *ctx, const float *host_som);
+/* Trainer<...,true>::update_som() (Trainer.h:306-309): device SOM -> host. */
+int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som);
+
+/* Trainer<...,true>::operator()(Data const&) (Trainer.h:263-304) applied to n_images
+ * images in order with sequential SOM semantics (image k+1 sees the weights left by
+ * image k, Pink/main_generic.h:87-89); n_images = 1 is exactly one operator() call.
+ * bmu_out (may be NULL) receives the best-matching neuron of each image, which the
+ * caller adds to m_update_info (Trainer.h:302-303). */
+int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out);
+/* Same with the images already on the device and the BMUs left on the device;
+ * asynchronous on the context's stream (see pink_hip_synchronize). */
+int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, uint32_t *dev_bmu_out);
+
+/* Mapper<...,true>::operator()(Data const&) (Mapper.h:181-208) for n_images images:
+ * heatmap_out[i*N + n] = sqrt(min over rotations of the distance), already square-rooted
+ * (Mapper.h:206); best_rot_out[i*N + n] = index of that rotation (may be NULL). */
+int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
+                 float *host_heatmap_out, uint32_t *host_best_rot_out);
+int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images,
+                        float *dev_heatmap_out, uint32_t *dev_best_rot_out);
+
+/* Wait for everything queued on the context's stream. */
+int pink_hip_synchronize(pink_hip_ctx *ctx);
+
+/* Debug taps used by the parity tests.
+ * pink_hip_rotate: SpatialTransformerGPU alone (CudaLib/generate_rotated_images.h:57-294):
+ *   variants_out holds R*C*D*D floats, variant k at ((k*C + c)*D + x)*D + y.
+ * pink_hip_distance: rotate + generate_euclidean_distance_matrix for one image against
+ *   the current SOM: dist_out[N] (float distance; integer modes: float(double(ssd)/factor^2)),
+ *   ssd_out[N] (exact integer sum, integer modes only; may be NULL), best_rot_out[N]. */
+int pink_hip_rotate(pink_hip_ctx *ctx, const float *host_image, float *host_variants_out);
+int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_dist_out,
+                      int64_t *host_ssd_out, uint32_t *host_best_rot_out);
+
+/* Number of elements in the distance region (incl. channels) as the context counts it. */
+uint32_t pink_hip_region_size(const pink_hip_ctx *ctx);
+
+/* Per-kernel timing with HIP events on the context's stream.  While enabled every
+ * launch of the rotation, distance and update kernels is bracketed by two events;
+ * pink_hip_kernel_times synchronises and returns, per kernel class, the number of
+ * launches and their summed duration in milliseconds since the last reset.
+ * Index: 0 rotation, 1 operand packing, 2 distance, 3 update, 4 finalise. */
+#define PINK_HIP_NUM_KERNEL_CLASSES 5
+int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable);
+int pink_hip_kernel_times(pink_hip_ctx *ctx, uint64_t *launches_out, double *ms_out);
+
+/* cuda_print_properties() / cuda_get_gpu_ids() (CudaLib/CudaLib.h:15-18): writes a
+ * one-line description of every visible device into buf; returns the device count
+ * or a negative status. */
+int pink_hip_device_info(char *buf, size_t len);
+
+/* Host-only helpers for the matrix a trainer context is created with: the loop in
+ * TrainerCommon's constructor (Trainer.h:69-76) over SOMLayout::get_distance
+ * (CartesianLayout.h:47-60,103-129 for 1/2/3 dimensions given as dims[0..ndims);
+ * HexagonalLayout.h:79-104 with dims[0] = the odd edge length) and one of the
+ * functors of UtilitiesLib/DistributionFunctor.cpp:19-59 (`sigma` is the step width
+ * for PINK_HIP_STEP).  factors_out holds N*N floats, N = pink_hip_som_size(...). */
+uint32_t pink_hip_som_size(uint32_t layout, const uint32_t *dims, uint32_t ndims);
+int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t ndims, uint32_t functor,
+                                 float sigma, float damping, float max_update_distance, float *factors_out);
+
+int pink_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,39 @@
+"""Compile the HIP library for gfx950 (cross-compiles without a GPU).
+
+    python -m pink_amd.build
+
+writes pink_amd/lib/libpink_hip.so.  The flags matter for parity with the CPU path:
+no floating-point contraction (products and sums of the rotation and update kernels
+round separately; the distance kernel asks for its fused multiply-add explicitly) and
+no packed-FP32 instructions.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SOURCES = [os.path.join(HERE, "csrc", "pink_hip.hip"), os.path.join(HERE, "csrc", "update_factors.cpp")]
+OUT = os.path.join(HERE, "lib", "libpink_hip.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-ffp-contract=off", "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+    "-I" + os.path.join(ROOT, "include"),
+]
+
+
+def build(verbose=False, extra=()):
+    os.makedirs(os.path.dirname(OUT), exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + list(extra) + SOURCES + ["-o", OUT]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return OUT
+
+
+if __name__ == "__main__":
+    build(verbose=True, extra=sys.argv[1:])

@@ -1,0 +1,970 @@
+// pink_hip.hip -- HIP kernels (gfx950) and the C ABI declared in include/pink_hip.h.
+//
+// One context = the device half of one reference Trainer<...,true> / Mapper<...,true>
+// (src/SelfOrganizingMapLib/Trainer.h:201-335, Mapper.h:129-230).  The kernels are
+// written for CDNA4: 64-lane wavefronts, lanes own rotations so that every global
+// access of the hot loop is a coalesced 256-byte row, neuron values arrive through
+// scalar loads, and the argmin over rotations is a packed 64-bit atomic minimum.
+//
+// Numerical contract (what the parity tests check against the CPU path):
+//   * rotated pixels: every product and sum rounded separately, in the order of
+//     ImageProcessingLib/rotate.h:37-63  -> bit-identical to the CPU;
+//   * float32 distance: one lane owns one (neuron, rotation) pair and accumulates
+//     fma(d, d, acc) over the region in the CPU's element order
+//     (ImageProcessingLib/euclidean_distance.h:47-100: the CPU squares in double and
+//     rounds the running sum to float at every step, which a fused multiply-add
+//     reproduces);
+//   * integer distance: exact sums of squared differences of quantised values;
+//   * update: w - ((w - x) * f), three roundings (SelfOrganizingMapLib/Trainer.h:175).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "pink_hip.h"
+
+namespace {
+
+constexpr uint32_t kWave = 64;
+constexpr uint32_t kEpadMultiple = 32;   // region length padded so k-loops need no tail
+constexpr int kClsRotate = 0, kClsPack = 1, kClsDist = 2, kClsUpdate = 3, kClsFinal = 4;
+
+thread_local std::string g_create_error;
+
+inline uint32_t round_up(uint32_t v, uint32_t m) { return (v + m - 1) / m * m; }
+
+// ---------------------------------------------------------------------------------
+// Device helpers
+// ---------------------------------------------------------------------------------
+
+__device__ __forceinline__ unsigned long long wave_min_u64(unsigned long long v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        unsigned long long o = __shfl_xor(v, off, 64);
+        v = o < v ? o : v;
+    }
+    return v;
+}
+
+// Value of base rotation `i` (angle i * 2pi / num_rot, 0 <= angle < 90 degrees) of one
+// channel at neuron pixel (x, y).  i == 0 is the centre crop / centre pad of
+// ImageProcessingLib/resize.h:15-40; i > 0 is ImageProcessingLib/rotate.h:31-65 with
+// the operation order kept (no contraction).
+__device__ __forceinline__ float base_pixel(const float *__restrict__ img, uint32_t I, uint32_t D,
+                                            uint32_t i, float cs, float sn, uint32_t x, uint32_t y)
+{
+    if (i == 0) {
+        if (I >= D) {
+            uint32_t m = (I - D) / 2;
+            return img[(size_t)(x + m) * I + (y + m)];
+        }
+        uint32_t m = (D - I) / 2;
+        uint32_t sx = x - m, sy = y - m;           // wraps for x < m: caught by the range test
+        return (sx < I && sy < I) ? img[(size_t)sx * I + sy] : 0.0f;
+    }
+    const float src_c = __fmul_rn((float)(I - 1), 0.5f);
+    const float dst_c = __fmul_rn((float)(D - 1), 0.5f);
+    const float px = __fsub_rn((float)x, dst_c);
+    const float py = __fsub_rn((float)y, dst_c);
+    const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+    const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+    const float lim = (float)(I - 1);
+    if (sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim) return 0.0f;
+    const uint32_t ix = (uint32_t)sxf, iy = (uint32_t)syf;
+    const float rx = __fsub_rn(sxf, (float)ix), ry = __fsub_rn(syf, (float)iy);
+    const float cx = __fsub_rn(1.0f, rx), cy = __fsub_rn(1.0f, ry);
+    // The neighbours one past the last row / column carry weight 0; clamp their index.
+    const uint32_t last = I * I - 1;
+    const uint32_t i00 = ix * I + iy;
+    const uint32_t i01 = min(i00 + 1, last);
+    const uint32_t i10 = min(i00 + I, last);
+    const uint32_t i11 = min(i00 + I + 1, last);
+    const float a = __fmul_rn(__fmul_rn(cx, cy), img[i00]);
+    const float b = __fmul_rn(__fmul_rn(cx, ry), img[i01]);
+    const float c = __fmul_rn(__fmul_rn(rx, cy), img[i10]);
+    const float d = __fmul_rn(__fmul_rn(rx, ry), img[i11]);
+    return __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
+}
+
+// ---------------------------------------------------------------------------------
+// Rotation: all num_rot * (flip ? 2 : 1) variants of a batch of images.
+// Block (i, c, b) computes base rotation i of channel c of image b once, keeps it in
+// LDS, and writes the 4 quarter turns and their flips as pure index permutations, each
+// variant row-major so that consecutive lanes store consecutive addresses.
+// Variant k = f * num_rot + q * (num_rot / 4) + i at rot[((b * R + k) * C + c) * D * D].
+// Quarter turn q of base B (ImageProcessingLib/rotate_90_degrees.h:15-26 applied q times):
+//   Q1[x][y] = B[D-1-y][x], Q2[x][y] = B[D-1-x][D-1-y], Q3[x][y] = B[y][D-1-x];
+// flip (ImageProcessingLib/flip.h:14-30): F[x][y] = V[D-1-x][y].
+// Block (0, 0, b) also resets the image's argmin keys.
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
+                                                const float *__restrict__ cos_t, const float *__restrict__ sin_t,
+                                                unsigned long long *__restrict__ key, uint32_t N,
+                                                uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
+                                                uint32_t use_flip, uint32_t use_lds)
+{
+    extern __shared__ float s_base[];
+    const uint32_t i = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
+    const uint32_t nrr = num_rot / 4;
+    const uint32_t R = num_rot * (use_flip ? 2u : 1u);
+    const uint32_t DD = D * D;
+    const float *img = images + ((size_t)b * C + c) * I * I;
+    float *out = rot + (size_t)b * R * C * DD;
+    const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
+    const uint32_t nq = num_rot == 1 ? 1u : 4u, nf = use_flip ? 2u : 1u;
+
+    if (i == 0 && c == 0)
+        for (uint32_t n = threadIdx.x; n < N; n += blockDim.x) key[(size_t)b * N + n] = ~0ull;
+
+    if (use_lds) {
+        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x)
+            s_base[p] = base_pixel(img, I, D, i, cs, sn, p / D, p % D);
+        __syncthreads();
+        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
+            const uint32_t x = p / D, y = p % D;
+            for (uint32_t f = 0; f < nf; ++f) {
+                const uint32_t xs = f ? D - 1 - x : x;
+                for (uint32_t q = 0; q < nq; ++q) {
+                    uint32_t a, bb;
+                    switch (q) {
+                    case 0: a = xs; bb = y; break;
+                    case 1: a = D - 1 - y; bb = xs; break;
+                    case 2: a = D - 1 - xs; bb = D - 1 - y; break;
+                    default: a = y; bb = D - 1 - xs; break;
+                    }
+                    const uint32_t k = f * num_rot + q * nrr + i;
+                    out[((size_t)k * C + c) * DD + p] = s_base[a * D + bb];
+                }
+            }
+        }
+    } else {
+        // Neurons too large for LDS: compute each base pixel once and scatter it.
+        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
+            const uint32_t a = p / D, bb = p % D;
+            const float v = base_pixel(img, I, D, i, cs, sn, a, bb);
+            for (uint32_t q = 0; q < nq; ++q) {
+                uint32_t x, y;
+                switch (q) {
+                case 0: x = a; y = bb; break;
+                case 1: x = bb; y = D - 1 - a; break;
+                case 2: x = D - 1 - a; y = D - 1 - bb; break;
+                default: x = D - 1 - bb; y = a; break;
+                }
+                for (uint32_t f = 0; f < nf; ++f) {
+                    const uint32_t xf = f ? D - 1 - x : x;
+                    const uint32_t k = f * num_rot + q * nrr + i;
+                    out[((size_t)k * C + c) * DD + xf * D + y] = v;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Operand packing for the vector-ALU distance kernels.
+//   somP[n][k]    = conv(som[n][off[k]])                      k < E, 0 beyond (row length Epad)
+//   rotT[b][k][r] = conv(rot[b][r][off[k]])   k-major so that the 64 lanes of a wave
+//                   (64 consecutive rotations) read one 256-byte row per k.
+// conv: float32 copy, or quantisation q = T(x * factor) saturated to [0, factor]
+// (CudaLib/copy_and_transform_kernel.h:27-28) held as int32.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ int32_t quantise(float x, float factor)
+{
+    const float v = __fmul_rn(x, factor);
+    if (!(v > 0.0f)) return 0;
+    if (v >= factor) return (int32_t)factor;
+    return (int32_t)v;
+}
+
+template <bool QUANT>
+__global__ __launch_bounds__(256) void k_pack_som(const float *__restrict__ som, const uint32_t *__restrict__ off,
+                                                  void *__restrict__ somP, uint32_t N, uint32_t S, uint32_t E,
+                                                  uint32_t Epad, float factor)
+{
+    const size_t total = (size_t)N * Epad;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t n = (uint32_t)(t / Epad), k = (uint32_t)(t % Epad);
+        const float v = k < E ? som[(size_t)n * S + off[k]] : 0.0f;
+        if (QUANT) ((int32_t *)somP)[t] = k < E ? quantise(v, factor) : 0;
+        else ((float *)somP)[t] = v;
+    }
+}
+
+template <bool QUANT>
+__global__ __launch_bounds__(256) void k_pack_rot(const float *__restrict__ rot, const uint32_t *__restrict__ off,
+                                                  void *__restrict__ rotT, uint32_t R, uint32_t S, uint32_t E,
+                                                  uint32_t Epad, uint32_t Rpad, float factor)
+{
+    __shared__ float tile[32][33];
+    const uint32_t b = blockIdx.z;
+    const uint32_t k0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+    for (uint32_t rr = ty; rr < 32; rr += 8) {
+        const uint32_t r = r0 + rr, k = k0 + tx;
+        tile[rr][tx] = (r < R && k < E) ? rot[((size_t)b * R + r) * S + off[k]] : 0.0f;
+    }
+    __syncthreads();
+    for (uint32_t kk = ty; kk < 32; kk += 8) {
+        const uint32_t k = k0 + kk, r = r0 + tx;
+        const float v = tile[tx][kk];
+        const size_t o = ((size_t)b * Epad + k) * Rpad + r;
+        if (QUANT) ((int32_t *)rotT)[o] = (r < R && k < E) ? quantise(v, factor) : 0;
+        else ((float *)rotT)[o] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Distance + argmin over rotations on the vector ALU.
+// One wave = 64 consecutive rotations x TN neurons.  Lane l owns rotation r0 + l and TN
+// accumulators; the neuron values of the k-loop are wave-uniform (scalar loads).  Each
+// (neuron, rotation) sum is accumulated sequentially over k by one lane -- no split-K, no
+// cross-lane partial sums -- so the float32 result has the CPU's rounding sequence.
+// The minimum over rotations is exact: a wave-level minimum of (value, rotation) keys,
+// then one 64-bit atomic minimum per neuron.  Key = value << shift | rotation, with
+// value = float bits (non-negative floats order like their bit patterns) or the integer sum.
+// MODE 0: float32, 1: uint8 (int32 sums), 2: uint16 (int64 sums).
+// ---------------------------------------------------------------------------------
+template <int MODE, int TN>
+__global__ __launch_bounds__(64) void k_dist_valu(const void *__restrict__ somP_, const void *__restrict__ rotT_,
+                                                  unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
+                                                  uint32_t R, uint32_t Rpad)
+{
+    using OpT = typename std::conditional<MODE == 0, float, int32_t>::type;
+    using AccT = typename std::conditional<MODE == 0, float, typename std::conditional<MODE == 1, int32_t, long long>::type>::type;
+    const OpT *__restrict__ somP = (const OpT *)somP_;
+    const OpT *__restrict__ rotT = (const OpT *)rotT_;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t r = blockIdx.x * kWave + lane;
+    const uint32_t n0 = blockIdx.y * TN;
+    const uint32_t b = blockIdx.z;
+    const OpT *rp = rotT + (size_t)b * Epad * Rpad + r;
+    const OpT *np[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad;
+
+    AccT acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = 0;
+
+    for (uint32_t k = 0; k < Epad; k += 8) {
+        OpT bv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) bv[u] = rp[(size_t)(k + u) * Rpad];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const OpT a = np[j][k + u];
+                if (MODE == 0) {
+                    const float d = __fsub_rn((float)a, (float)bv[u]);
+                    acc[j] = (AccT)__builtin_fmaf(d, d, (float)acc[j]);
+                } else {
+                    const int32_t d = (int32_t)a - (int32_t)bv[u];
+                    acc[j] += (AccT)d * (AccT)d;
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        unsigned long long kv;
+        if (MODE == 0) kv = ((unsigned long long)__float_as_uint((float)acc[j]) << 32) | r;
+        else kv = ((unsigned long long)acc[j] << 16) | r;
+        if (r >= R) kv = ~0ull;
+        kv = wave_min_u64(kv);
+        if (lane == 0 && n0 + j < N) atomicMin(&key[(size_t)b * N + n0 + j], kv);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
+// Every block recomputes the best-matching neuron from the N keys (first minimum wins),
+// then block (part, n) pulls its slice of neuron n toward that neuron's best variant:
+//   w = w - ((w - x) * f),  f = factors[bmu * N + n], skipped when f == 0.
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const float *__restrict__ rot,
+                                                const unsigned long long *__restrict__ key,
+                                                const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
+                                                uint32_t N, uint32_t S, uint32_t parts, uint32_t shift)
+{
+    __shared__ unsigned long long s_val[256];
+    __shared__ uint32_t s_idx[256];
+    const uint32_t tid = threadIdx.x;
+    unsigned long long bv = ~0ull;
+    uint32_t bi = 0xffffffffu;
+    for (uint32_t n = tid; n < N; n += 256) {
+        const unsigned long long v = key[n] >> shift;
+        if (v < bv) { bv = v; bi = n; }        // ascending n per thread: first minimum kept
+    }
+    s_val[tid] = bv;
+    s_idx[tid] = bi;
+    __syncthreads();
+    for (uint32_t s = 128; s > 0; s >>= 1) {
+        if (tid < s) {
+            const unsigned long long ov = s_val[tid + s];
+            const uint32_t oi = s_idx[tid + s];
+            if (ov < s_val[tid] || (ov == s_val[tid] && oi < s_idx[tid])) { s_val[tid] = ov; s_idx[tid] = oi; }
+        }
+        __syncthreads();
+    }
+    const uint32_t bmu = s_idx[0];
+    const uint32_t n = blockIdx.y, part = blockIdx.x;
+    if (n == 0 && part == 0 && tid == 0) *bmu_out = bmu;
+
+    const float f = factors[(size_t)bmu * N + n];
+    if (f == 0.0f) return;
+    const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
+    const float *__restrict__ x = rot + (size_t)r * S;
+    float *__restrict__ w = som + (size_t)n * S;
+    const uint32_t chunk = (S + parts - 1) / parts;
+    const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
+    for (uint32_t j = j0 + tid; j < j1; j += 256) {
+        const float wv = w[j];
+        w[j] = __fsub_rn(wv, __fmul_rn(__fsub_rn(wv, x[j]), f));
+    }
+}
+
+// Decode keys: distance (optionally square-rooted for the mapper, Mapper.h:206), exact
+// integer sum, best rotation.  Integer modes: distance = float(double(ssd) / factor^2).
+__global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__restrict__ key, float *__restrict__ dist,
+                                                  long long *__restrict__ ssd, uint32_t *__restrict__ best,
+                                                  size_t total, uint32_t shift, uint32_t is_int, double factor2,
+                                                  uint32_t do_sqrt)
+{
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    const unsigned long long kv = key[t];
+    const unsigned long long v = kv >> shift;
+    float d;
+    if (is_int) {
+        d = (float)((double)(long long)v / factor2);
+        if (ssd) ssd[t] = (long long)v;
+    } else {
+        d = __uint_as_float((uint32_t)v);
+    }
+    // sqrt in double, then one rounding: the correctly rounded float square root
+    // (std::sqrt(float) on the host, Mapper.h:206)
+    if (do_sqrt) d = (float)sqrt((double)d);
+    if (dist) dist[t] = d;
+    if (best) best[t] = (uint32_t)(kv & ((1ull << shift) - 1ull));
+}
+
+// ---------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------
+struct EventPair { hipEvent_t a, b; int cls; };
+
+}  // namespace
+
+struct pink_hip_ctx {
+    pink_hip_config cfg{};
+    uint32_t N = 0, C = 0, I = 0, D = 0, S = 0, R = 0, nrr = 0, E = 0, Epad = 0, Rpad = 0;
+    uint32_t isz = 0;          // floats per image
+    uint32_t Bcap = 1;         // images per launch group
+    uint32_t shift = 32;       // key = value << shift | rotation
+    uint32_t factor = 1;       // 255 / 65535 in the integer modes
+    bool trainer = false;
+    bool use_lds = true;
+    int device = 0;
+    hipStream_t stream = nullptr;
+
+    float *d_som = nullptr, *d_rot = nullptr, *d_cos = nullptr, *d_sin = nullptr, *d_factors = nullptr;
+    uint32_t *d_region = nullptr;
+    unsigned long long *d_key = nullptr;
+    void *d_somP = nullptr, *d_rotT = nullptr;
+    uint32_t *d_bmu_scratch = nullptr;
+    float *d_dist = nullptr;
+    long long *d_ssd = nullptr;
+    uint32_t *d_best = nullptr;
+
+    bool profiling = false;
+    std::vector<EventPair> events;
+    std::vector<hipEvent_t> event_pool;
+    uint64_t prof_launches[PINK_HIP_NUM_KERNEL_CLASSES] = {0};
+    double prof_ms[PINK_HIP_NUM_KERNEL_CLASSES] = {0};
+
+    std::string err;
+};
+
+namespace {
+
+int fail(pink_hip_ctx *ctx, int code, const std::string &msg)
+{
+    if (ctx) ctx->err = msg;
+    else g_create_error = msg;
+    return code;
+}
+
+#define HIP_TRY(ctx, call)                                                                          \
+    do {                                                                                            \
+        hipError_t e_ = (call);                                                                     \
+        if (e_ != hipSuccess)                                                                       \
+            return fail(ctx, e_ == hipErrorOutOfMemory ? PINK_HIP_ENOMEM : PINK_HIP_EDEVICE,        \
+                        std::string(#call) + ": " + hipGetErrorString(e_));                         \
+    } while (0)
+
+struct Timed {
+    pink_hip_ctx *ctx;
+    int cls;
+    hipEvent_t a = nullptr, b = nullptr;
+    Timed(pink_hip_ctx *c, int k) : ctx(c), cls(k)
+    {
+        if (!ctx->profiling) return;
+        auto take = [&]() {
+            hipEvent_t e = nullptr;
+            if (!ctx->event_pool.empty()) { e = ctx->event_pool.back(); ctx->event_pool.pop_back(); }
+            else if (hipEventCreate(&e) != hipSuccess) e = nullptr;
+            return e;
+        };
+        a = take();
+        b = take();
+        if (a) (void)hipEventRecord(a, ctx->stream);
+    }
+    ~Timed()
+    {
+        if (!ctx->profiling || !a || !b) return;
+        (void)hipEventRecord(b, ctx->stream);
+        ctx->events.push_back({a, b, cls});
+    }
+};
+
+int drain_events(pink_hip_ctx *ctx)
+{
+    if (ctx->events.empty()) return PINK_HIP_OK;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (auto &p : ctx->events) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+            ctx->prof_ms[p.cls] += ms;
+            ctx->prof_launches[p.cls] += 1;
+        }
+        ctx->event_pool.push_back(p.a);
+        ctx->event_pool.push_back(p.b);
+    }
+    ctx->events.clear();
+    return PINK_HIP_OK;
+}
+
+// Offsets of the distance region inside one C*D*D neuron, in the CPU's summation order.
+// Quadratic: ImageProcessingLib/euclidean_distance.h:47-100.  Circular:
+// ImageProcessingLib/circular_euclidean_distance.h:37-88 -- including its integer
+// radius e/2, the empty last row of an odd diameter (NaN radicand) and, for
+// multi-channel data, the missing channel offset (channel 0 counted C times).
+std::vector<uint32_t> build_region(uint32_t C, uint32_t D, uint32_t e, uint32_t shape)
+{
+    std::vector<uint32_t> off;
+    if (shape == PINK_HIP_QUADRATIC) {
+        const uint32_t beg = static_cast<uint32_t>((D - e) * 0.5);
+        for (uint32_t c = 0; c < C; ++c)
+            for (uint32_t i = beg; i < beg + e; ++i)
+                for (uint32_t j = beg; j < beg + e; ++j) off.push_back(c * D * D + i * D + j);
+    } else {
+        const uint32_t center = D / 2, radius = e / 2;
+        for (uint32_t c = 0; c < C; ++c)
+            for (uint32_t i = 0; i < e; ++i) {
+                const double delta = std::sqrt(2 * radius * (i + 0.5) - std::pow(i + 0.5, 2));
+                if (std::isnan(delta)) continue;
+                const uint32_t gi = i + (D - e) / 2;
+                const double hi = std::round(center + delta);
+                for (uint32_t j = static_cast<uint32_t>(std::round(center - delta)); j < hi; ++j)
+                    off.push_back(gi * D + j);
+            }
+    }
+    return off;
+}
+
+template <typename T>
+int dev_alloc(pink_hip_ctx *ctx, T **p, size_t count)
+{
+    HIP_TRY(ctx, hipMalloc((void **)p, (count ? count : 1) * sizeof(T)));
+    return PINK_HIP_OK;
+}
+
+#define TRY(expr)                         \
+    do {                                  \
+        int rc_ = (expr);                 \
+        if (rc_ != PINK_HIP_OK) return rc_; \
+    } while (0)
+
+int launch_check(pink_hip_ctx *ctx, const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(ctx, PINK_HIP_EDEVICE, std::string(what) + ": " + hipGetErrorString(e));
+    return PINK_HIP_OK;
+}
+
+bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT; }
+
+// --- launch groups ---------------------------------------------------------------
+
+int run_pack_som(pink_hip_ctx *ctx)
+{
+    Timed t(ctx, kClsPack);
+    const size_t total = (size_t)ctx->N * ctx->Epad;
+    const uint32_t blocks = (uint32_t)std::min<size_t>((total + 255) / 256, 8192);
+    if (is_int(ctx))
+        hipLaunchKernelGGL(k_pack_som<true>, dim3(blocks), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+                           ctx->d_somP, ctx->N, ctx->S, ctx->E, ctx->Epad, (float)ctx->factor);
+    else
+        hipLaunchKernelGGL(k_pack_som<false>, dim3(blocks), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+                           ctx->d_somP, ctx->N, ctx->S, ctx->E, ctx->Epad, 1.0f);
+    return launch_check(ctx, "k_pack_som");
+}
+
+int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
+{
+    Timed t(ctx, kClsRotate);
+    const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
+    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->D * sizeof(float) : 0;
+    hipLaunchKernelGGL(k_rotate, grid, dim3(256), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin,
+                       ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,
+                       ctx->use_lds ? 1u : 0u);
+    return launch_check(ctx, "k_rotate");
+}
+
+int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
+{
+    Timed t(ctx, kClsPack);
+    const dim3 grid(ctx->Epad / 32, ctx->Rpad / 32, B);
+    if (is_int(ctx))
+        hipLaunchKernelGGL(k_pack_rot<true>, grid, dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region, ctx->d_rotT,
+                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, (float)ctx->factor);
+    else
+        hipLaunchKernelGGL(k_pack_rot<false>, grid, dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region, ctx->d_rotT,
+                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, 1.0f);
+    return launch_check(ctx, "k_pack_rot");
+}
+
+template <int MODE>
+void launch_dist(pink_hip_ctx *ctx, uint32_t B)
+{
+    // Neurons per wave: as many as keep at least ~2 waves per SIMD in flight.
+    const uint32_t rblocks = ctx->Rpad / kWave;
+    const size_t target_waves = 2048;
+    uint32_t tn = 8;
+    while (tn > 1 && (size_t)rblocks * ((ctx->N + tn - 1) / tn) * B < target_waves) tn >>= 1;
+    const dim3 grid(rblocks, (ctx->N + tn - 1) / tn, B);
+#define LAUNCH_TN(T_)                                                                                           \
+    hipLaunchKernelGGL((k_dist_valu<MODE, T_>), grid, dim3(64), 0, ctx->stream, ctx->d_somP, ctx->d_rotT, ctx->d_key, \
+                       ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    switch (tn) {
+    case 8: LAUNCH_TN(8); break;
+    case 4: LAUNCH_TN(4); break;
+    case 2: LAUNCH_TN(2); break;
+    default: LAUNCH_TN(1); break;
+    }
+#undef LAUNCH_TN
+}
+
+int run_dist(pink_hip_ctx *ctx, uint32_t B)
+{
+    Timed t(ctx, kClsDist);
+    switch (ctx->cfg.ed_type) {
+    case PINK_HIP_FLOAT: launch_dist<0>(ctx, B); break;
+    case PINK_HIP_UINT8: launch_dist<1>(ctx, B); break;
+    default: launch_dist<2>(ctx, B); break;
+    }
+    return launch_check(ctx, "k_dist");
+}
+
+int run_update(pink_hip_ctx *ctx, uint32_t *dev_bmu_out)
+{
+    Timed t(ctx, kClsUpdate);
+    uint32_t parts = (1024 + ctx->N - 1) / ctx->N;
+    parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
+    hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_rot, ctx->d_key,
+                       ctx->d_factors, dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift);
+    return launch_check(ctx, "k_update");
+}
+
+int run_finalize(pink_hip_ctx *ctx, uint32_t B, float *dev_dist, long long *dev_ssd, uint32_t *dev_best, bool do_sqrt)
+{
+    Timed t(ctx, kClsFinal);
+    const size_t total = (size_t)B * ctx->N;
+    const double f2 = (double)ctx->factor * (double)ctx->factor;
+    hipLaunchKernelGGL(k_finalize, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, ctx->stream, ctx->d_key,
+                       dev_dist, dev_ssd, dev_best, total, ctx->shift, is_int(ctx) ? 1u : 0u, f2, do_sqrt ? 1u : 0u);
+    return launch_check(ctx, "k_finalize");
+}
+
+int free_all(pink_hip_ctx *ctx)
+{
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    for (auto &p : ctx->events) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+    for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+    void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
+                    ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best};
+    for (void *p : bufs) if (p) (void)hipFree(p);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    return PINK_HIP_OK;
+}
+
+int init_ctx(pink_hip_ctx *ctx)
+{
+    const pink_hip_config &c = ctx->cfg;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
+
+    // Rotation tables: cos/sin of i * 2pi/num_rot in float, as the CPU evaluates them
+    // (SelfOrganizingMapLib/generate_rotated_images.h:69,94; ImageProcessingLib/rotate.h:20-21).
+    std::vector<float> cs(std::max(ctx->nrr, 1u), 1.0f), sn(std::max(ctx->nrr, 1u), 0.0f);
+    const float angle_step = static_cast<float>(2 * M_PI) / c.num_rot;
+    for (uint32_t i = 1; i < ctx->nrr; ++i) {
+        const float alpha = i * angle_step;
+        cs[i] = std::cos(alpha);
+        sn[i] = std::sin(alpha);
+    }
+    TRY(dev_alloc(ctx, &ctx->d_cos, cs.size()));
+    TRY(dev_alloc(ctx, &ctx->d_sin, sn.size()));
+    HIP_TRY(ctx, hipMemcpy(ctx->d_cos, cs.data(), cs.size() * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(ctx, hipMemcpy(ctx->d_sin, sn.data(), sn.size() * sizeof(float), hipMemcpyHostToDevice));
+
+    const std::vector<uint32_t> region = build_region(ctx->C, ctx->D, c.ed_dim, c.ed_shape);
+    ctx->E = (uint32_t)region.size();
+    if (ctx->E == 0) return fail(ctx, PINK_HIP_EINVAL, "Euclidean distance region is empty");
+    ctx->Epad = round_up(ctx->E, kEpadMultiple);
+    ctx->Rpad = round_up(ctx->R, kWave);
+    if (is_int(ctx)) {
+        // key = ssd << 16 | rotation: the sum must stay below 2^48 and R below 2^16.
+        const double max_ssd = (double)ctx->factor * ctx->factor * ctx->E;
+        if (ctx->R > 65536 || max_ssd >= 281474976710656.0 || (c.ed_type == PINK_HIP_UINT8 && max_ssd >= 2147483648.0))
+            return fail(ctx, PINK_HIP_EINVAL, "distance region or rotation count too large for the integer distance modes");
+    }
+    TRY(dev_alloc(ctx, &ctx->d_region, region.size()));
+    HIP_TRY(ctx, hipMemcpy(ctx->d_region, region.data(), region.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+
+    // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
+    const size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
+    if (ctx->trainer) ctx->Bcap = 1;
+    else {
+        size_t b = c.max_batch ? c.max_batch : 256;
+        const size_t budget = (size_t)4 << 30;
+        while (b > 1 && b * per_image > budget) b >>= 1;
+        ctx->Bcap = (uint32_t)b;
+    }
+    const size_t B = ctx->Bcap;
+    ctx->use_lds = (size_t)ctx->D * ctx->D * sizeof(float) <= 64 * 1024;
+
+    TRY(dev_alloc(ctx, &ctx->d_som, (size_t)ctx->N * ctx->S));
+    HIP_TRY(ctx, hipMemset(ctx->d_som, 0, (size_t)ctx->N * ctx->S * sizeof(float)));
+    TRY(dev_alloc(ctx, &ctx->d_rot, B * ctx->R * ctx->S));
+    TRY(dev_alloc(ctx, &ctx->d_key, B * ctx->N));
+    TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad));
+    TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
+    TRY(dev_alloc(ctx, &ctx->d_bmu_scratch, 1));
+    TRY(dev_alloc(ctx, &ctx->d_dist, B * ctx->N));
+    TRY(dev_alloc(ctx, &ctx->d_ssd, B * ctx->N));
+    TRY(dev_alloc(ctx, &ctx->d_best, B * ctx->N));
+    if (ctx->trainer) {
+        TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
+        HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
+                               hipMemcpyHostToDevice));
+    }
+    HIP_TRY(ctx, hipDeviceSynchronize());   // set-up copies ran on the null stream
+    TRY(run_pack_som(ctx));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return PINK_HIP_OK;
+}
+
+// rotate -> pack -> distance for B images already on the device; keys left in d_key.
+int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
+{
+    TRY(run_rotate(ctx, dev_images, B));
+    TRY(run_pack_rot(ctx, B));
+    TRY(run_dist(ctx, B));
+    return PINK_HIP_OK;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------
+extern "C" {
+
+int pink_hip_abi_version(void) { return PINK_HIP_ABI_VERSION; }
+
+const char *pink_hip_last_error(const pink_hip_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
+
+int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
+{
+    if (!out || !cfg) return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: null argument");
+    *out = nullptr;
+    // SelfOrganizingMapLib/Trainer.h:66-67, Mapper.h:59-62
+    if (cfg->num_rot == 0 || (cfg->num_rot != 1 && cfg->num_rot % 4 != 0))
+        return fail(nullptr, PINK_HIP_EINVAL, "Number of rotations must be 1 or larger then 1 and divisible by 4");
+    // SelfOrganizingMapLib/Mapper.h:63-66
+    if (cfg->ed_dim > cfg->neuron_dim)
+        return fail(nullptr, PINK_HIP_EINVAL, "Euclidean distance dimension larger than neuron dimension");
+    // CudaLib/generate_rotated_images.h:119-121 (only bilinear interpolation exists on the device)
+    if (cfg->num_rot > 4 && cfg->interpolation != PINK_HIP_BILINEAR)
+        return fail(nullptr, PINK_HIP_EINVAL, "generate_rotated_images: unknown interpolation type");
+    if (cfg->som_size == 0 || cfg->channels == 0 || cfg->image_dim == 0 || cfg->neuron_dim == 0 || cfg->ed_dim == 0)
+        return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: zero-sized SOM, image, neuron or distance region");
+    if (cfg->ed_type > PINK_HIP_UINT8 || cfg->ed_shape > PINK_HIP_CIRCULAR)
+        return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: unknown distance type or shape");
+    if ((uint64_t)cfg->image_dim * cfg->image_dim >= (1ull << 31) ||
+        (uint64_t)cfg->channels * cfg->neuron_dim * cfg->neuron_dim >= (1ull << 31))
+        return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: image or neuron too large");
+
+    pink_hip_ctx *ctx = new (std::nothrow) pink_hip_ctx();
+    if (!ctx) return fail(nullptr, PINK_HIP_ENOMEM, "pink_hip_create: out of host memory");
+    ctx->cfg = *cfg;
+    ctx->N = cfg->som_size;
+    ctx->C = cfg->channels;
+    ctx->I = cfg->image_dim;
+    ctx->D = cfg->neuron_dim;
+    ctx->S = cfg->channels * cfg->neuron_dim * cfg->neuron_dim;
+    ctx->isz = cfg->channels * cfg->image_dim * cfg->image_dim;
+    ctx->R = cfg->num_rot * (cfg->use_flip ? 2u : 1u);
+    ctx->nrr = cfg->num_rot / 4;
+    ctx->trainer = cfg->update_factors != nullptr;
+    ctx->device = cfg->device;
+    ctx->factor = cfg->ed_type == PINK_HIP_UINT8 ? 255u : cfg->ed_type == PINK_HIP_UINT16 ? 65535u : 1u;
+    ctx->shift = cfg->ed_type == PINK_HIP_FLOAT ? 32u : 16u;
+
+    int rc = init_ctx(ctx);
+    if (rc != PINK_HIP_OK) {
+        g_create_error = ctx->err;
+        free_all(ctx);
+        delete ctx;
+        return rc;
+    }
+    ctx->cfg.update_factors = nullptr;   // the host matrix is not kept
+    *out = ctx;
+    return PINK_HIP_OK;
+}
+
+void pink_hip_destroy(pink_hip_ctx *ctx)
+{
+    if (!ctx) return;
+    free_all(ctx);
+    delete ctx;
+}
+
+int pink_hip_synchronize(pink_hip_ctx *ctx)
+{
+    if (!ctx) return PINK_HIP_EINVAL;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return PINK_HIP_OK;
+}
+
+int pink_hip_set_som(pink_hip_ctx *ctx, const float *host_som)
+{
+    if (!ctx || !host_som) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_set_som: null argument");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemcpyAsync(ctx->d_som, host_som, (size_t)ctx->N * ctx->S * sizeof(float), hipMemcpyHostToDevice,
+                                ctx->stream));
+    TRY(run_pack_som(ctx));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return PINK_HIP_OK;
+}
+
+int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som)
+{
+    if (!ctx || !host_som) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_get_som: null argument");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemcpyAsync(host_som, ctx->d_som, (size_t)ctx->N * ctx->S * sizeof(float), hipMemcpyDeviceToHost,
+                                ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return PINK_HIP_OK;
+}
+
+int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, uint32_t *dev_bmu_out)
+{
+    if (!ctx || (!dev_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train_device: null argument");
+    if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_train: context was created without update factors");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    for (uint32_t i = 0; i < n_images; ++i) {
+        TRY(distance_group(ctx, dev_images + (size_t)i * ctx->isz, 1));
+        TRY(run_update(ctx, dev_bmu_out ? dev_bmu_out + i : ctx->d_bmu_scratch));
+        TRY(run_pack_som(ctx));
+    }
+    return PINK_HIP_OK;
+}
+
+int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out)
+{
+    if (!ctx || (!host_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train: null argument");
+    if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_train: context was created without update factors");
+    if (n_images == 0) return PINK_HIP_OK;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    // Stage the images in chunks of at most ~1 GiB.
+    const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
+    const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
+    float *d_img = nullptr;
+    uint32_t *d_bmu = nullptr;
+    HIP_TRY(ctx, hipMalloc((void **)&d_img, chunk * img_bytes));
+    if (hipMalloc((void **)&d_bmu, chunk * sizeof(uint32_t)) != hipSuccess) {
+        (void)hipFree(d_img);
+        return fail(ctx, PINK_HIP_ENOMEM, "pink_hip_train: device allocation failed");
+    }
+    int rc = PINK_HIP_OK;
+    for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += chunk) {
+        const uint32_t n = std::min(chunk, n_images - done);
+        hipError_t e = hipMemcpyAsync(d_img, host_images + (size_t)done * ctx->isz, n * img_bytes, hipMemcpyHostToDevice,
+                                      ctx->stream);
+        if (e == hipSuccess) rc = pink_hip_train_device(ctx, d_img, n, d_bmu);
+        if (e == hipSuccess && rc == PINK_HIP_OK && host_bmu_out)
+            e = hipMemcpyAsync(host_bmu_out + done, d_bmu, n * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess && rc == PINK_HIP_OK) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) rc = fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_train: ") + hipGetErrorString(e));
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(d_img);
+    (void)hipFree(d_bmu);
+    return rc;
+}
+
+int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, float *dev_heatmap_out,
+                        uint32_t *dev_best_rot_out)
+{
+    if (!ctx || (n_images && (!dev_images || !dev_heatmap_out)))
+        return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device: null argument");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    for (uint32_t done = 0; done < n_images; done += ctx->Bcap) {
+        const uint32_t B = std::min(ctx->Bcap, n_images - done);
+        TRY(distance_group(ctx, dev_images + (size_t)done * ctx->isz, B));
+        TRY(run_finalize(ctx, B, dev_heatmap_out + (size_t)done * ctx->N, nullptr,
+                         dev_best_rot_out ? dev_best_rot_out + (size_t)done * ctx->N : nullptr, true));
+    }
+    return PINK_HIP_OK;
+}
+
+int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, float *host_heatmap_out,
+                 uint32_t *host_best_rot_out)
+{
+    if (!ctx || (n_images && (!host_images || !host_heatmap_out)))
+        return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map: null argument");
+    if (n_images == 0) return PINK_HIP_OK;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
+    const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
+    float *d_img = nullptr, *d_heat = nullptr;
+    uint32_t *d_best = nullptr;
+    hipError_t e = hipMalloc((void **)&d_img, chunk * img_bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_heat, (size_t)chunk * ctx->N * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc((void **)&d_best, (size_t)chunk * ctx->N * sizeof(uint32_t));
+    int rc = e == hipSuccess ? PINK_HIP_OK : fail(ctx, PINK_HIP_ENOMEM, "pink_hip_map: device allocation failed");
+    for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += chunk) {
+        const uint32_t n = std::min(chunk, n_images - done);
+        e = hipMemcpyAsync(d_img, host_images + (size_t)done * ctx->isz, n * img_bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) rc = pink_hip_map_device(ctx, d_img, n, d_heat, d_best);
+        if (e == hipSuccess && rc == PINK_HIP_OK)
+            e = hipMemcpyAsync(host_heatmap_out + (size_t)done * ctx->N, d_heat, (size_t)n * ctx->N * sizeof(float),
+                               hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess && rc == PINK_HIP_OK && host_best_rot_out)
+            e = hipMemcpyAsync(host_best_rot_out + (size_t)done * ctx->N, d_best, (size_t)n * ctx->N * sizeof(uint32_t),
+                               hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess && rc == PINK_HIP_OK) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) rc = fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_map: ") + hipGetErrorString(e));
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (d_img) (void)hipFree(d_img);
+    if (d_heat) (void)hipFree(d_heat);
+    if (d_best) (void)hipFree(d_best);
+    return rc;
+}
+
+int pink_hip_rotate(pink_hip_ctx *ctx, const float *host_image, float *host_variants_out)
+{
+    if (!ctx || !host_image || !host_variants_out) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_rotate: null argument");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    float *d_img = nullptr;
+    HIP_TRY(ctx, hipMalloc((void **)&d_img, (size_t)ctx->isz * sizeof(float)));
+    hipError_t e = hipMemcpyAsync(d_img, host_image, (size_t)ctx->isz * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    int rc = PINK_HIP_OK;
+    if (e == hipSuccess) rc = run_rotate(ctx, d_img, 1);
+    if (e == hipSuccess && rc == PINK_HIP_OK)
+        e = hipMemcpyAsync(host_variants_out, ctx->d_rot, (size_t)ctx->R * ctx->S * sizeof(float), hipMemcpyDeviceToHost,
+                           ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(d_img);
+    if (e != hipSuccess) return fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_rotate: ") + hipGetErrorString(e));
+    return rc;
+}
+
+int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_dist_out, int64_t *host_ssd_out,
+                      uint32_t *host_best_rot_out)
+{
+    if (!ctx || !host_image) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_distance: null argument");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    float *d_img = nullptr;
+    HIP_TRY(ctx, hipMalloc((void **)&d_img, (size_t)ctx->isz * sizeof(float)));
+    hipError_t e = hipMemcpyAsync(d_img, host_image, (size_t)ctx->isz * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    int rc = PINK_HIP_OK;
+    if (e == hipSuccess) rc = distance_group(ctx, d_img, 1);
+    if (e == hipSuccess && rc == PINK_HIP_OK) rc = run_finalize(ctx, 1, ctx->d_dist, ctx->d_ssd, ctx->d_best, false);
+    const size_t n = ctx->N;
+    if (e == hipSuccess && rc == PINK_HIP_OK && host_dist_out)
+        e = hipMemcpyAsync(host_dist_out, ctx->d_dist, n * sizeof(float), hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess && rc == PINK_HIP_OK && host_ssd_out && is_int(ctx))
+        e = hipMemcpyAsync(host_ssd_out, ctx->d_ssd, n * sizeof(long long), hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess && rc == PINK_HIP_OK && host_best_rot_out)
+        e = hipMemcpyAsync(host_best_rot_out, ctx->d_best, n * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(d_img);
+    if (e != hipSuccess) return fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_distance: ") + hipGetErrorString(e));
+    return rc;
+}
+
+uint32_t pink_hip_region_size(const pink_hip_ctx *ctx) { return ctx ? ctx->E : 0; }
+
+int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)
+{
+    if (!ctx) return PINK_HIP_EINVAL;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    TRY(drain_events(ctx));
+    ctx->profiling = enable != 0;
+    for (int i = 0; i < PINK_HIP_NUM_KERNEL_CLASSES; ++i) { ctx->prof_launches[i] = 0; ctx->prof_ms[i] = 0.0; }
+    return PINK_HIP_OK;
+}
+
+int pink_hip_kernel_times(pink_hip_ctx *ctx, uint64_t *launches_out, double *ms_out)
+{
+    if (!ctx) return PINK_HIP_EINVAL;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    TRY(drain_events(ctx));
+    for (int i = 0; i < PINK_HIP_NUM_KERNEL_CLASSES; ++i) {
+        if (launches_out) launches_out[i] = ctx->prof_launches[i];
+        if (ms_out) ms_out[i] = ctx->prof_ms[i];
+    }
+    return PINK_HIP_OK;
+}
+
+int pink_hip_device_info(char *buf, size_t len)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) {
+        g_create_error = std::string("hipGetDeviceCount: ") + hipGetErrorString(e);
+        return PINK_HIP_EDEVICE;
+    }
+    std::string s;
+    for (int d = 0; d < count; ++d) {
+        hipDeviceProp_t p;
+        if (hipGetDeviceProperties(&p, d) != hipSuccess) continue;
+        char line[512];
+        snprintf(line, sizeof line, "device %d: %s (%s), %d CUs, %d MHz, %.1f GiB, LDS/block %zu KiB\n", d, p.name,
+                 p.gcnArchName, p.multiProcessorCount, p.clockRate / 1000, p.totalGlobalMem / 1073741824.0,
+                 p.sharedMemPerBlock / 1024);
+        s += line;
+    }
+    if (buf && len) {
+        strncpy(buf, s.c_str(), len - 1);
+        buf[len - 1] = '\0';
+    }
+    return count;
+}
+
+}  // extern "C"

@@ -1,0 +1,239 @@
+"""GPU parity: the HIP path through the C ABI against the CPU oracle.
+
+Bars (stated where checked): rotated pixels bit-exact; float32 distances bit-exact
+with the oracle (stricter than the 1e-5 relative gate) and best rotation / BMU
+identical; integer sums, best rotations and BMUs bit-exact; trained weights
+bit-exact after several sequential images (gate: 1e-4 absolute).
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import oracle as O
+from pink_amd import capi, synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+ROT_SHAPES = [
+    # C, I, D, num_rot, flip
+    (1, 64, 44, 360, True), (1, 150, 106, 360, True), (3, 100, 70, 180, True), (1, 28, 28, 4, True),
+    (1, 64, 45, 360, True), (1, 64, 100, 360, True), (1, 124, 91, 360, True), (2, 17, 24, 16, False),
+    (1, 2, 4, 1, False), (1, 4, 2, 8, True), (1, 5, 3, 360, False), (3, 9, 9, 1, True),
+    (1, 200, 141, 8, True),     # 141*141*4 B > 64 KiB: the no-LDS path
+]
+
+
+@pytest.mark.parametrize("C_,I,D,nrot,flip", ROT_SHAPES)
+def test_rotate_bit_exact(C_, I, D, nrot, flip):
+    say("rotate", C_, I, D, nrot, flip)
+    rng = np.random.default_rng(I * 1000 + D + nrot)
+    img = rng.random((C_, I, I), dtype=np.float32)
+    with capi.Context(3, C_, I, D, nrot, flip, min(D, 2)) as ctx:
+        got = ctx.rotate(img)
+    want = O.rotated_images(img, C_, I, D, nrot, flip)
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_rotate_reference_golden():
+    # test/SelfOrganizingMapTest/generate_rotated_images.cpp:15-41
+    with capi.Context(1, 1, 2, 2, 4, False, 2) as ctx:
+        out = ctx.rotate(np.array([1, 2, 3, 4], np.float32))
+    assert out.ravel().tolist() == [1, 2, 3, 4, 3, 1, 4, 2, 4, 3, 2, 1, 2, 4, 1, 3]
+    with capi.Context(1, 2, 2, 2, 4, False, 2) as ctx:
+        out = ctx.rotate(np.arange(1, 9, dtype=np.float32))
+    assert out.ravel().tolist() == [1, 2, 3, 4, 5, 6, 7, 8, 3, 1, 4, 2, 7, 5, 8, 6,
+                                    4, 3, 2, 1, 8, 7, 6, 5, 2, 4, 1, 3, 6, 8, 5, 7]
+
+
+DIST_SHAPES = [
+    # N, C, I, D, nrot, flip, ed, shape
+    (100, 1, 64, 44, 360, True, 32, capi.QUADRATIC),      # cfg 0 / 1
+    (64, 1, 28, 28, 4, True, 28, capi.QUADRATIC),         # cfg 4
+    (37, 1, 40, 29, 16, True, 21, capi.CIRCULAR),
+    (9, 2, 17, 24, 8, False, 13, capi.QUADRATIC),
+    (9, 2, 17, 24, 8, True, 13, capi.CIRCULAR),           # 3-D circular: channel 0 counted twice (CPU rule)
+    (4, 1, 8, 8, 1, False, 8, capi.QUADRATIC),
+    (5, 1, 8, 8, 1, True, 5, capi.QUADRATIC),
+    (331, 1, 150, 106, 360, True, 75, capi.CIRCULAR),     # cfg 2
+    (1600, 3, 100, 70, 180, True, 50, capi.QUADRATIC),    # cfg 3
+]
+
+
+def _som_and_image(N, C_, I, D, seed):
+    rng = np.random.default_rng(seed)
+    som = rng.random((N, C_ * D * D), dtype=np.float32)
+    img = rng.random((C_, I, I), dtype=np.float32)
+    return som, img
+
+
+@pytest.mark.parametrize("ed_type", [capi.FLOAT, capi.UINT8, capi.UINT16])
+@pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_", DIST_SHAPES)
+def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
+    if N >= 331 and ed_type != {331: capi.UINT16, 1600: capi.FLOAT}[N]:
+        pytest.skip("large shapes run in their configured mode only (oracle time)")
+    say("distance", N, C_, I, D, nrot, flip, ed, shape_, ed_type)
+    som, img = _som_and_image(N, C_, I, D, N + D + ed)
+    if N < 331:
+        som[1] = O.rotated_images(img, C_, I, D, nrot, flip)[min(3, nrot - 1)].ravel()   # an exact match
+        som[2] = som[1] * np.float32(0.5)
+    with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type) as ctx:
+        ctx.set_som(som)
+        assert ctx.region_size == len(O.region(C_, D, ed, shape_))
+        d, ssd, best = ctx.distance(img)
+    s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, ed_type)
+    rot = O.rotated_images(img, C_, I, D, nrot, flip)
+    od, ossd, obest = O.distance_matrix(s, som, rot)
+    if ed_type == capi.FLOAT:
+        # gate: 1e-5 relative, argmin identical up to ties; achieved and asserted: bit-exact
+        assert np.array_equal(bits(d), bits(od))
+    else:
+        assert np.array_equal(ssd, ossd)
+        assert np.array_equal(bits(d), bits(od))
+    assert np.array_equal(best, obest)
+
+
+TRAIN_CASES = [
+    # workload, images, ed_type override
+    ("cfg0", 6, None), ("cfg4", 40, None), ("cfg0", 4, capi.UINT8), ("cfg2", 2, None), ("cfg3", 1, None),
+]
+
+
+@pytest.mark.parametrize("name,n,ed_type", TRAIN_CASES)
+def test_train_parity(name, n, ed_type):
+    w = synthetic.WORKLOADS[name]
+    ed_type = w.ed_type if ed_type is None else ed_type
+    say("train", name, n, ed_type)
+    imgs = synthetic.images(w, n)
+    som0 = synthetic.initial_som(w)
+    F = synthetic.update_factors(w)
+    with capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                      w.ed_shape, ed_type, F) as ctx:
+        ctx.set_som(som0)
+        bmu = ctx.train(imgs)
+        got = ctx.get_som()
+    s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                w.ed_shape, ed_type)
+    want = som0.copy()
+    obmu = O.train(s, want, imgs, F)
+    assert np.array_equal(bmu, obmu)
+    # gate: 1e-4 absolute (test/CudaTest/compare_trainer_cpu.cu:76); asserted: bit-exact
+    assert np.abs(got - want).max() <= 1e-4
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_train_one_call_per_image_equals_batched_call():
+    w = synthetic.WORKLOADS["cfg4"]
+    imgs = synthetic.images(w, 12)
+    som0 = synthetic.initial_som(w)
+    with synthetic.make_context(w) as a, synthetic.make_context(w) as b:
+        a.set_som(som0)
+        b.set_som(som0)
+        bm_a = a.train(imgs)
+        bm_b = np.concatenate([b.train(imgs[i]) for i in range(len(imgs))])
+        assert np.array_equal(bm_a, bm_b)
+        assert np.array_equal(bits(a.get_som()), bits(b.get_som()))
+
+
+def test_reference_trainer_known_answers():
+    # test/SelfOrganizingMapTest/Trainer.cpp:49-94 and test/CudaTest/update_neurons.cu:16-41
+    F = capi.make_update_factors(capi.CARTESIAN, [2, 2], capi.GAUSSIAN, 1.1, 0.2, 0.0)
+    with capi.Context(4, 1, 2, 2, 1, False, 2, update_factors=F) as ctx:
+        ctx.set_som(np.zeros((4, 4), np.float32))
+        ctx.train(np.array([1000, 2000, 3000, 4000], np.float32))
+        assert int(ctx.get_som()[0, 3]) == 290
+    F = capi.make_update_factors(capi.CARTESIAN, [1, 1], capi.STEP, 10.0)
+    with capi.Context(1, 1, 4, 2, 1, False, 2, update_factors=F) as ctx:
+        ctx.set_som(np.zeros((1, 4), np.float32))
+        ctx.train(np.arange(1, 17, dtype=np.float32))
+        assert ctx.get_som().ravel().tolist() == [6, 7, 10, 11]
+    F = capi.make_update_factors(capi.CARTESIAN, [2, 2], capi.STEP, 0.0)
+    with capi.Context(4, 2, 2, 2, 4, False, 2, update_factors=F) as ctx:
+        som = np.zeros((4, 8), np.float32)
+        som[1] = [4, 3, 2, 1, 8, 7, 6, 5]
+        ctx.set_som(som)
+        bmu = ctx.train(np.arange(1, 9, dtype=np.float32))
+        assert bmu.tolist() == [1] and np.array_equal(ctx.get_som(), som)
+
+
+MAP_CASES = [("cfg1", 24, None), ("cfg0", 5, capi.FLOAT), ("cfg4", 300, None), ("cfg2", 2, None)]
+
+
+@pytest.mark.parametrize("name,n,ed_type", MAP_CASES)
+def test_map_parity(name, n, ed_type):
+    w = synthetic.WORKLOADS[name]
+    ed_type = w.ed_type if ed_type is None else ed_type
+    say("map", name, n, ed_type)
+    imgs = synthetic.images(w, n)
+    som = synthetic.initial_som(w)
+    som[3] = O.rotated_images(imgs[1], w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip)[5 % w.R].ravel()
+    with capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                      w.ed_shape, ed_type, None, max_batch=7) as ctx:
+        ctx.set_som(som)
+        heat, best = ctx.map(imgs)
+    s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                w.ed_shape, ed_type)
+    oheat, obest = O.map_images(s, som, imgs)
+    assert np.array_equal(bits(heat), bits(oheat))
+    assert np.array_equal(best, obest)
+
+
+def test_reference_mapper_known_answers():
+    # test/CudaTest/mapper.cu:115-119 in float, uint8 and uint16; circular_ed.cu:23-53
+    for som_dim, nd, idim, ed, nrot, flip in [(1, 2, 2, 2, 1, False), (1, 3, 3, 2, 1, False), (1, 3, 3, 2, 360, False),
+                                              (2, 3, 3, 2, 360, False), (2, 3, 3, 2, 360, True)]:
+        N = som_dim * som_dim
+        for ed_type in (capi.FLOAT, capi.UINT8, capi.UINT16):
+            with capi.Context(N, 1, idim, nd, nrot, flip, ed, capi.QUADRATIC, ed_type) as ctx:
+                ctx.set_som(np.ones((N, nd * nd), np.float32))
+                heat, _ = ctx.map(np.zeros((idim, idim), np.float32))
+            assert heat.ravel().tolist() == [2.0] * N
+    image = np.zeros(16, np.float32)
+    image[4] = 1.0
+    som = np.zeros(64, np.float32)
+    som[4], som[18], som[43], som[61] = 1.0, 0.5, 0.8, 0.3
+    with capi.Context(4, 1, 4, 4, 4, False, 4, capi.CIRCULAR, capi.FLOAT) as ctx:
+        ctx.set_som(som)
+        heat, best = ctx.map(image)
+    assert np.allclose(heat.ravel(), [0.0, 0.5, 0.2, 0.7], atol=0.01)
+    assert best.ravel().tolist() == [0, 1, 2, 3]
+
+
+def test_map_full_size_properties():
+    """cfg 1 at a size the oracle does not cover: properties that hold at any size."""
+    w = synthetic.WORKLOADS["cfg1"]
+    n = 2000
+    imgs = synthetic.images(w, n)
+    som = synthetic.initial_som(w)
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(som)
+        heat, best = ctx.map(imgs)
+        heat2, best2 = ctx.map(imgs[::-1])
+        # rotating an image by a quarter turn permutes its variants: same heatmap, shifted index
+        turned = np.ascontiguousarray(np.rot90(imgs[:50], k=-1, axes=(2, 3)))
+        heat3, best3 = ctx.map(turned)
+    assert np.array_equal(bits(heat2[::-1]), bits(heat)) and np.array_equal(best2[::-1], best)   # order-independent
+    assert (heat >= 0).all() and np.isfinite(heat).all() and (best < w.R).all()
+    assert np.array_equal(bits(heat3), bits(heat[:50]))
+
+
+def test_profiling_counts_launches():
+    w = synthetic.WORKLOADS["cfg4"]
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(synthetic.initial_som(w))
+        ctx.set_profiling(True)
+        ctx.train(synthetic.images(w, 5))
+        t = ctx.kernel_times()
+        ctx.set_profiling(False)
+    assert t["rotate"][0] == 5 and t["distance"][0] == 5 and t["update"][0] == 5
+    assert all(ms >= 0 for _, ms in t.values())
