@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the PINK hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1]
+
+A step is one pass of the hot path over one batch of synthetic input: the whole
+image set of the workload, mapped (cfg1) or trained in order (cfg0/2/3/4), with the
+images already resident in HBM when the timed region starts.  Default workload: cfg1
+(mapping 20 000 images, uint8 distances, 720 variants) with the SOM obtained by
+training cfg0 for one epoch on the GPU first (untimed).
+
+Prints ONE JSON line with the throughput, a `roofline` object for the kernel class
+that takes most of the time (durations from HIP events recorded on the library's own
+stream around every launch) and a `cpu_baseline` object (the CPU oracle timed on a
+bounded sample of the same workload on this host's cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+FP32_PEAK_TFLOPS = 157.3       # MI355X vector fp32 (packed FMA), published
+
+DTYPE_NAME = {0: "f32", 1: "u16", 2: "u8"}
+
+
+def algorithmic_per_image(w, E):
+    """Algorithmic bytes / operations per image for each kernel class."""
+    elem = {0: 4, 1: 2, 2: 1}[w.ed_type]
+    S, R, N = w.neuron_size, w.R, w.som_size
+    return {
+        # write all variants once, read the image once
+        "rotate": {"bytes": R * S * 4 + w.image_size * 4},
+        # region of every variant read as float32 and written in the distance type
+        "pack": {"bytes": R * E * (4 + elem)},
+        # every operand element read once; one subtract-square-accumulate = 2 operations
+        "distance": {"bytes": (R + N) * E * elem, "ops": 2 * N * R * E},
+        # SOM read + written, one variant read per neuron
+        "update": {"bytes": 3 * N * S * 4},
+        "finalize": {"bytes": N * 16},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every figure is a "
+              "single-MI355X figure)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from pink_amd import capi, synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    w = synthetic.WORKLOADS[args.workload]
+    n_images = args.images or w.n_images
+    kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA}[args.kernel]
+
+    t0 = time.time()
+    imgs_host = synthetic.images(w, n_images)
+    som0 = synthetic.initial_som(w)
+    if w.mode == "map":
+        # the SOM of cfg0 after one epoch, trained here on the GPU (set-up, not timed)
+        w0 = synthetic.WORKLOADS["cfg0"]
+        with synthetic.make_context(w0) as tr:
+            tr.set_som(som0)
+            tr.train(synthetic.images(w0))
+            som0 = tr.get_som()
+    setup_s = time.time() - t0
+
+    ctx = synthetic.make_context(w, kernel_choice=kernel_choice)
+    E = ctx.region_size
+    ctx.set_som(som0)
+    d_imgs = torch.from_numpy(imgs_host).to(dev)
+    d_heat = torch.empty((n_images, w.som_size), dtype=torch.float32, device=dev)
+    d_best = torch.empty((n_images, w.som_size), dtype=torch.int32, device=dev)
+    d_bmu = torch.empty((n_images,), dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+
+    def step():
+        if w.mode == "map":
+            ctx.map_device(d_imgs.data_ptr(), n_images, d_heat.data_ptr(), d_best.data_ptr())
+        else:
+            ctx.train_device(d_imgs.data_ptr(), n_images, d_bmu.data_ptr())
+
+    for _ in range(args.warmup):
+        if w.mode == "train":
+            ctx.set_som(som0)
+        step()
+    ctx.synchronize()
+
+    # ---- timed region: exactly `steps` steps, HIP events around every kernel launch ----
+    if w.mode == "train":
+        ctx.set_som(som0)
+    profile_in_timed = w.mode == "map"          # a few hundred launches: event cost is nil
+    ctx.set_profiling(profile_in_timed)
+    torch.cuda.synchronize()
+    ctx.synchronize()
+    t_start = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t_start
+    if profile_in_timed:
+        times = ctx.kernel_times()
+        prof_images = n_images * args.steps
+    else:
+        # training issues thousands of launches per second: per-kernel events go in their own pass
+        prof_images = min(n_images, 256)
+        ctx.set_profiling(True)
+        ctx.train_device(d_imgs.data_ptr(), prof_images, d_bmu.data_ptr())
+        times = ctx.kernel_times()
+    ctx.set_profiling(False)
+
+    value = n_images * args.steps / elapsed
+    alg = algorithmic_per_image(w, E)
+    total_ms = sum(ms for _, ms in times.values()) or 1e-9
+    dominant = max(times, key=lambda k: times[k][1])
+    launches, ms = times[dominant]
+    avg_ms = ms / max(launches, 1)
+    imgs_per_launch = prof_images / max(launches, 1)
+    if dominant == "distance" and w.ed_type == capi.FLOAT:
+        # direct float32 form: sub + fma per pair element on the vector ALU, 2 ops counted per pair
+        bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
+        achieved = alg["distance"]["ops"] * imgs_per_launch / (avg_ms * 1e-3) / 1e12
+    else:
+        bound, unit, peak = "hbm", "GB/s", HBM_PEAK_GBS
+        achieved = alg[dominant]["bytes"] * imgs_per_launch / (avg_ms * 1e-3) / 1e9
+    roofline = {
+        "kernel": dominant, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+        "frac": round(achieved / peak, 5), "traffic": None,
+        "avg_launch_ms": round(avg_ms, 6), "launches": launches, "images_per_launch": imgs_per_launch,
+        "measured": "timed region" if profile_in_timed else "separate pass of %d images" % prof_images,
+        "share_of_kernel_time": round(ms / total_ms, 4),
+        "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
+    }
+    if "ops" in alg[dominant] and w.ed_type != capi.FLOAT:
+        roofline["mfma_int8_frac"] = round(
+            alg[dominant]["ops"] * imgs_per_launch / (avg_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 5)
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle as O
+        s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                    w.ed_shape, w.ed_type)
+        F = synthetic.update_factors(w) if w.mode == "train" else None
+
+        def cpu_run(n):
+            t = time.perf_counter()
+            if w.mode == "map":
+                O.map_images(s, som0, imgs_host[:n])
+            else:
+                O.train(s, som0.copy(), imgs_host[:n], F)
+            return time.perf_counter() - t
+
+        cpu_run(min(2, n_images))                      # warm-up
+        probe_n = min(4, n_images)
+        probe = cpu_run(probe_n)
+        n_cpu = int(max(probe_n, min(n_images, 12.0 / max(probe / probe_n, 1e-6))))
+        dt = cpu_run(n_cpu)
+        cpu = {"value": round(n_cpu / dt, 3), "unit": "images/s", "cores": O.num_threads(), "kind": "port",
+               "sample": "%d images of %s, %.1f s, OpenMP over rotations" % (n_cpu, w.name, dt)}
+
+    out = {
+        "metric": ("map" if w.mode == "map" else "train") + " images/sec @%d rot x flip" % w.R,
+        "value": round(value, 2), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": DTYPE_NAME[w.ed_type], "data": "synthetic",
+        "config": {"workload": w.name, "mode": w.mode, "images_per_step": n_images, "som_size": w.som_size,
+                   "neuron": [w.channels, w.neuron_dim, w.neuron_dim], "image": [w.channels, w.image_dim, w.image_dim],
+                   "variants": w.R, "region_elements": E, "distance_kernel": args.kernel,
+                   "som": "cfg0 trained 1 epoch on the GPU" if w.mode == "map" else "mt19937(1234) U[0,1)"},
+        "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(setup_s, 2),
+    }
+    ctx.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -228,6 +228,10 @@ def map_images(s, som, images):
     return heat, best
 
 
+def num_threads():
+    return int(lib().pink_oracle_num_threads())
+
+
 def fill_random_uniform(n, seed):
     a = np.empty(n, np.float32)
     lib().pink_oracle_fill_random_uniform(_p(a, C.c_float), C.c_size_t(n), C.c_uint32(seed))

@@ -11,6 +11,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #ifndef M_PI
 #define M_PI 3.14159265358979323846
 #endif
@@ -587,4 +591,14 @@ void pink_oracle_fill_random_uniform(float *a, size_t length, uint32_t seed)
         if (v >= 1.0f) v = nextafterf(1.0f, 0.0f);
         a[i] = v;
     }
+}
+
+/* Threads the OpenMP loops above will use (1 without OpenMP). */
+int pink_oracle_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
 }

@@ -122,6 +122,8 @@ int pink_oracle_map(const pink_oracle_shape *s, const float *som, const float *i
 void pink_oracle_fill_random_uniform(float *a, size_t length, uint32_t seed);
 void pink_oracle_mt19937_raw(uint32_t seed, uint32_t *out, size_t n);
 
+int pink_oracle_num_threads(void);
+
 #ifdef __cplusplus
 }
 #endif
