@@ -284,6 +284,207 @@ __global__ __launch_bounds__(64) void k_dist_valu(const void *__restrict__ somP_
     }
 }
 
+
+// ---------------------------------------------------------------------------------
+// uint8 distance on the matrix cores (mapping).
+//
+// Integer sums are order-independent, so the uint8 distance is recast exactly as
+//   ssd(n, r) = |a'_n|^2 + |b'_r|^2 - 2 a'_n . b'_r,    x' = q(x) - 128 in [-128, 127],
+// with the dot products on v_mfma_i32_32x32x32_i8 (int32 accumulation, exact).
+//
+// Operand layout ("fragment-major"): rows in tiles of 32, k in steps of 32; one
+// (tile, k-step) fragment is 1 KiB = 64 lanes x 16 bytes, lane l holding row l % 32,
+// k = kstep * 32 + (l / 32) * 16 .. + 16.  A wave loads a fragment with one fully
+// coalesced 16-byte-per-lane access and feeds it to the MFMA unchanged.  Both operands
+// use the same layout, so the k assignment inside a fragment cancels out.
+//
+// Rotation operand rows are ordered (base rotation i, symmetry) instead of by variant
+// index: row = i * 8 + flip * 4 + quarter.  The 8 symmetries of a base rotation are
+// then adjacent, one block owns whole fragments, and the true variant index
+// k = flip * num_rot + quarter * (num_rot / 4) + i travels in the argmin key, so ties
+// still resolve to the lowest variant index.
+// ---------------------------------------------------------------------------------
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// Rotation + quantisation + packing, no float variants written.  Block (tile, b): base
+// rotations 4*tile .. 4*tile+3 of image b are evaluated only at the pixels some region
+// element of some symmetry refers to (`need`), quantised and shifted into LDS; every
+// operand byte is then a gather through the precomputed table
+//   poff[sym][e] = position in the base rotation of region element e of symmetry sym
+// (position S = a zero byte, used for the padding beyond E).
+__global__ __launch_bounds__(256) void k_rotpack_u8(const float *__restrict__ images, v4i *__restrict__ Pb,
+                                                    int *__restrict__ nb, const float *__restrict__ cos_t,
+                                                    const float *__restrict__ sin_t,
+                                                    const unsigned short *__restrict__ poff,
+                                                    const uint32_t *__restrict__ need, uint32_t n_need, uint32_t C,
+                                                    uint32_t I, uint32_t D, uint32_t S, uint32_t num_rot,
+                                                    uint32_t use_flip, uint32_t nrr_eff, uint32_t KS, uint32_t RT)
+{
+    extern __shared__ signed char s_q[];              // 4 * (S + 1) quantised pixels, then 32 ints
+    const uint32_t tile = blockIdx.x, b = blockIdx.y;
+    const uint32_t stride = S + 1;
+    int *s_nb = (int *)(s_q + ((4 * stride + 15) & ~15u));
+    const uint32_t DD = D * D;
+    const float *img = images + (size_t)b * C * I * I;
+
+    if (threadIdx.x < 32) s_nb[threadIdx.x] = 0;
+    if (threadIdx.x < 4) s_q[threadIdx.x * stride + S] = 0;
+    for (uint32_t t = threadIdx.x; t < 4 * n_need; t += blockDim.x) {
+        const uint32_t g = t / n_need, p = need[t % n_need];
+        const uint32_t i = tile * 4 + g;
+        signed char v = 0;
+        if (i < nrr_eff) {
+            const uint32_t c = p / DD, px = (p % DD) / D, py = p % D;
+            const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
+            v = (signed char)(quantise(base_pixel(img + (size_t)c * I * I, I, D, i, cs, sn, px, py), 255.0f) - 128);
+        }
+        s_q[g * stride + p] = v;
+    }
+    __syncthreads();
+
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = lane & 31, half = lane >> 5;
+    const uint32_t g = row >> 3, sym = row & 7;
+    const uint32_t Kp = KS * 32;
+    const signed char *src = s_q + g * stride;
+    const unsigned short *tab = poff + (size_t)sym * Kp + half * 16;
+    int sq = 0;
+    for (uint32_t ks = wave; ks < KS; ks += 4) {
+        const unsigned short *tp = tab + ks * 32;
+        v4i frag;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int v = src[tp[w4 * 4 + u]];
+                sq += v * v;
+                word |= (uint32_t)(v & 0xff) << (8 * u);
+            }
+            frag[w4] = (int)word;
+        }
+        Pb[(((size_t)b * RT + tile) * KS + ks) * 64 + lane] = frag;
+    }
+    atomicAdd(&s_nb[row], sq);
+    __syncthreads();
+    if (threadIdx.x < 32) nb[((size_t)b * RT + tile) * 32 + threadIdx.x] = s_nb[threadIdx.x];
+}
+
+// SOM operand in the same fragment-major layout plus |a'_n|^2.  One block per neuron.
+__global__ __launch_bounds__(256) void k_pack_som_u8(const float *__restrict__ som, const uint32_t *__restrict__ off,
+                                                     signed char *__restrict__ Pa, int *__restrict__ na, uint32_t N,
+                                                     uint32_t S, uint32_t E, uint32_t KS)
+{
+    __shared__ int s_sum[256];
+    const uint32_t n = blockIdx.x;      // 0 .. NT*32-1, rows beyond N are zero
+    const uint32_t Kp = KS * 32;
+    int sq = 0;
+    for (uint32_t k = threadIdx.x; k < Kp; k += 256) {
+        int v = 0;
+        if (n < N && k < E) v = quantise(som[(size_t)n * S + off[k]], 255.0f) - 128;
+        sq += v * v;
+        const uint32_t lane = (n & 31) + 32 * ((k & 31) >> 4);
+        Pa[((((size_t)(n >> 5) * KS + (k >> 5)) * 64 + lane) << 4) + (k & 15)] = (signed char)v;
+    }
+    s_sum[threadIdx.x] = sq;
+    __syncthreads();
+    for (uint32_t s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) s_sum[threadIdx.x] += s_sum[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) na[n] = s_sum[0];
+}
+
+// Distance + argmin.  The whole SOM operand stays in LDS; a block walks over images, its
+// 8 waves share the rotation tiles of one image.  Per (tile, k-step) a wave loads one
+// rotation fragment from HBM (each byte of the operand is read exactly once) and issues NT
+// MFMAs against the neuron fragments in LDS.  Rotations are the MFMA's row operand, so a
+// lane ends up with 16 rotations of ONE neuron (column lane % 32) per accumulator set: the
+// minimum over rotations is a running in-lane minimum, one shuffle across the two
+// half-waves, and one LDS pass across the 8 waves -- no atomics.
+template <int NT>
+__global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa, const int *__restrict__ na,
+                                                      const v4i *__restrict__ Pb, const int *__restrict__ nb,
+                                                      unsigned long long *__restrict__ key, uint32_t N, uint32_t KS,
+                                                      uint32_t RT, uint32_t B, uint32_t num_rot, uint32_t use_flip,
+                                                      uint32_t nrr_eff)
+{
+    extern __shared__ v4i s_a[];                                   // NT * KS * 64 fragments' lanes
+    unsigned long long *s_key = (unsigned long long *)(s_a + (size_t)NT * KS * 64);   // 8 waves x NT*32
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t col = lane & 31, half = lane >> 5;
+    const uint32_t nrr = num_rot / 4;
+
+    for (uint32_t t = threadIdx.x; t < NT * KS * 64; t += blockDim.x) s_a[t] = Pa[t];
+    int na_l[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) na_l[nt] = na[nt * 32 + col];
+    __syncthreads();
+
+    for (uint32_t b = blockIdx.x; b < B; b += gridDim.x) {
+        unsigned long long best[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) best[nt] = ~0ull;
+
+        for (uint32_t rt = wave; rt < RT; rt += 8) {
+            v16i acc[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) acc[nt][j] = 0;
+            const v4i *pb = Pb + ((size_t)b * RT + rt) * KS * 64 + lane;
+            for (uint32_t ks = 0; ks < KS; ks += 8) {
+                v4i bf[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) bf[u] = pb[(size_t)min(ks + u, KS - 1) * 64];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (ks + u < KS) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+                            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u], s_a[((size_t)nt * KS + ks + u) * 64 + lane],
+                                                                            acc[nt], 0, 0, 0);
+                    }
+                }
+            }
+            // accumulator j of lane l: rotation row 8*(j/4) + 4*(l/32) + j%4 of the tile, neuron column l%32
+            const int *nbp = nb + ((size_t)b * RT + rt) * 32;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const uint32_t ib = j >> 2, q = j & 3;
+                const uint32_t i = rt * 4 + ib;
+                const bool valid = i < nrr_eff && (num_rot != 1 || q == 0) && (use_flip || half == 0);
+                const uint32_t k = half * num_rot + q * nrr + i;
+                const int nbv = nbp[8 * ib + 4 * half + q];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int ssd = na_l[nt] + nbv - 2 * acc[nt][j];
+                    const unsigned long long kv = valid ? (((unsigned long long)(uint32_t)ssd << 16) | k) : ~0ull;
+                    best[nt] = kv < best[nt] ? kv : best[nt];
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const unsigned long long o = __shfl_xor(best[nt], 32, 64);
+            best[nt] = o < best[nt] ? o : best[nt];
+            if (half == 0) s_key[wave * (NT * 32) + nt * 32 + col] = best[nt];
+        }
+        __syncthreads();
+        if (threadIdx.x < NT * 32) {
+            unsigned long long m = s_key[threadIdx.x];
+#pragma unroll
+            for (int w = 1; w < 8; ++w) {
+                const unsigned long long o = s_key[w * (NT * 32) + threadIdx.x];
+                m = o < m ? o : m;
+            }
+            if (threadIdx.x < N) key[(size_t)b * N + threadIdx.x] = m;
+        }
+        __syncthreads();
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
 // Every block recomputes the best-matching neuron from the N keys (first minimum wins),
@@ -384,6 +585,16 @@ struct pink_hip_ctx {
     float *d_dist = nullptr;
     long long *d_ssd = nullptr;
     uint32_t *d_best = nullptr;
+
+    // uint8 mapping on the matrix cores
+    bool mfma = false;
+    uint32_t KS = 0, RT = 0, NT = 0, n_need = 0, nrr_eff = 1;
+    size_t lds_dist = 0, lds_rotpack = 0;
+    int num_cu = 256;
+    signed char *d_Pa = nullptr, *d_Pb = nullptr;
+    int *d_na = nullptr, *d_nb = nullptr;
+    unsigned short *d_poff = nullptr;
+    uint32_t *d_need = nullptr;
 
     bool profiling = false;
     std::vector<EventPair> events;
@@ -508,6 +719,11 @@ bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT
 int run_pack_som(pink_hip_ctx *ctx)
 {
     Timed t(ctx, kClsPack);
+    if (ctx->mfma) {
+        hipLaunchKernelGGL(k_pack_som_u8, dim3(ctx->NT * 32), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+                           ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->E, ctx->KS);
+        return launch_check(ctx, "k_pack_som_u8");
+    }
     const size_t total = (size_t)ctx->N * ctx->Epad;
     const uint32_t blocks = (uint32_t)std::min<size_t>((total + 255) / 256, 8192);
     if (is_int(ctx))
@@ -602,7 +818,8 @@ int free_all(pink_hip_ctx *ctx)
     for (auto &p : ctx->events) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
-                    ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best};
+                    ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
+                    ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -642,11 +859,67 @@ int init_ctx(pink_hip_ctx *ctx)
     TRY(dev_alloc(ctx, &ctx->d_region, region.size()));
     HIP_TRY(ctx, hipMemcpy(ctx->d_region, region.data(), region.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
 
+    // uint8 mapping on the matrix cores: SOMs of up to 128 neurons whose packed operand fits in LDS.
+    {
+        hipDeviceProp_t prop;
+        HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
+        ctx->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        const size_t lds_max = std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024) - 1024;
+        ctx->nrr_eff = std::max(ctx->nrr, 1u);
+        ctx->KS = ctx->Epad / 32;
+        ctx->NT = (ctx->N + 31) / 32;
+        ctx->RT = (ctx->nrr_eff + 3) / 4;
+        ctx->lds_dist = (size_t)ctx->NT * ctx->KS * 1024 + (size_t)8 * ctx->NT * 32 * 8;
+        ctx->lds_rotpack = (((size_t)4 * (ctx->S + 1) + 15) & ~(size_t)15) + 32 * sizeof(int);
+        const bool fits = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && ctx->N <= 128 && ctx->S + 1 <= 65535 &&
+                          ctx->lds_dist <= lds_max && ctx->lds_rotpack <= lds_max;
+        if (c.kernel_choice == PINK_HIP_KERNEL_MFMA && !fits)
+            return fail(ctx, PINK_HIP_EINVAL, "the MFMA distance kernel needs a uint8 mapper with at most 128 neurons "
+                                              "whose packed SOM fits in LDS");
+        ctx->mfma = fits && c.kernel_choice != PINK_HIP_KERNEL_VALU;
+    }
+    if (ctx->mfma) {
+        // poff[sym][e]: where region element e of symmetry sym = flip*4 + quarter sits in the base rotation.
+        const uint32_t D = ctx->D, DD = D * D, Kp = ctx->KS * 32;
+        std::vector<unsigned short> poff((size_t)8 * Kp, (unsigned short)ctx->S);
+        std::vector<char> used(ctx->S, 0);
+        for (uint32_t sym = 0; sym < 8; ++sym) {
+            const uint32_t f = sym >> 2, q = sym & 3;
+            const bool sym_valid = (c.num_rot != 1 || q == 0) && (c.use_flip || f == 0);
+            for (uint32_t e = 0; e < ctx->E; ++e) {
+                const uint32_t ch = region[e] / DD, x = (region[e] % DD) / D, y = region[e] % D;
+                const uint32_t xs = f ? D - 1 - x : x;
+                uint32_t a, bb;
+                switch (q) {
+                case 0: a = xs; bb = y; break;
+                case 1: a = D - 1 - y; bb = xs; break;
+                case 2: a = D - 1 - xs; bb = D - 1 - y; break;
+                default: a = y; bb = D - 1 - xs; break;
+                }
+                const uint32_t p = ch * DD + a * D + bb;
+                if (sym_valid) { poff[(size_t)sym * Kp + e] = (unsigned short)p; used[p] = 1; }
+            }
+        }
+        std::vector<uint32_t> need;
+        for (uint32_t p = 0; p < ctx->S; ++p) if (used[p]) need.push_back(p);
+        ctx->n_need = (uint32_t)need.size();
+        TRY(dev_alloc(ctx, &ctx->d_poff, poff.size()));
+        TRY(dev_alloc(ctx, &ctx->d_need, need.size()));
+        HIP_TRY(ctx, hipMemcpy(ctx->d_poff, poff.data(), poff.size() * sizeof(unsigned short), hipMemcpyHostToDevice));
+        HIP_TRY(ctx, hipMemcpy(ctx->d_need, need.data(), need.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotpack_u8, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)ctx->lds_rotpack));
+        const void *fn = ctx->NT == 1 ? (const void *)k_dist_mfma_u8<1> : ctx->NT == 2 ? (const void *)k_dist_mfma_u8<2>
+                       : ctx->NT == 3 ? (const void *)k_dist_mfma_u8<3> : (const void *)k_dist_mfma_u8<4>;
+        HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_dist));
+    }
+
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
-    const size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
+    size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
+    if (ctx->mfma) per_image = (size_t)ctx->RT * ctx->KS * 1024 + (size_t)ctx->RT * 128 + (size_t)ctx->N * 24;
     if (ctx->trainer) ctx->Bcap = 1;
     else {
-        size_t b = c.max_batch ? c.max_batch : 256;
+        size_t b = c.max_batch ? c.max_batch : (ctx->mfma ? 2048 : 256);
         const size_t budget = (size_t)4 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
         ctx->Bcap = (uint32_t)b;
@@ -656,10 +929,19 @@ int init_ctx(pink_hip_ctx *ctx)
 
     TRY(dev_alloc(ctx, &ctx->d_som, (size_t)ctx->N * ctx->S));
     HIP_TRY(ctx, hipMemset(ctx->d_som, 0, (size_t)ctx->N * ctx->S * sizeof(float)));
-    TRY(dev_alloc(ctx, &ctx->d_rot, B * ctx->R * ctx->S));
+    // The float variants are only materialised per launch group on the vector-ALU path; the
+    // matrix-core path keeps room for one image (pink_hip_rotate).
+    TRY(dev_alloc(ctx, &ctx->d_rot, (ctx->mfma ? 1 : B) * ctx->R * ctx->S));
     TRY(dev_alloc(ctx, &ctx->d_key, B * ctx->N));
-    TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad));
-    TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
+    if (ctx->mfma) {
+        TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->NT * ctx->KS * 1024));
+        TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->NT * 32));
+        TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RT * ctx->KS * 1024));
+        TRY(dev_alloc(ctx, &ctx->d_nb, B * ctx->RT * 32));
+    } else {
+        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad));
+        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
+    }
     TRY(dev_alloc(ctx, &ctx->d_bmu_scratch, 1));
     TRY(dev_alloc(ctx, &ctx->d_dist, B * ctx->N));
     TRY(dev_alloc(ctx, &ctx->d_ssd, B * ctx->N));
@@ -676,8 +958,41 @@ int init_ctx(pink_hip_ctx *ctx)
 }
 
 // rotate -> pack -> distance for B images already on the device; keys left in d_key.
+int run_rotpack_mfma(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
+{
+    Timed t(ctx, kClsRotate);
+    hipLaunchKernelGGL(k_rotpack_u8, dim3(ctx->RT, B), dim3(256), ctx->lds_rotpack, ctx->stream, dev_images,
+                       (v4i *)ctx->d_Pb, ctx->d_nb, ctx->d_cos, ctx->d_sin, ctx->d_poff, ctx->d_need, ctx->n_need,
+                       ctx->C, ctx->I, ctx->D, ctx->S, ctx->cfg.num_rot, ctx->cfg.use_flip, ctx->nrr_eff, ctx->KS,
+                       ctx->RT);
+    return launch_check(ctx, "k_rotpack_u8");
+}
+
+int run_dist_mfma(pink_hip_ctx *ctx, uint32_t B)
+{
+    Timed t(ctx, kClsDist);
+    const dim3 grid(std::min<uint32_t>(B, (uint32_t)ctx->num_cu));
+#define LAUNCH_NT(T_)                                                                                              \
+    hipLaunchKernelGGL((k_dist_mfma_u8<T_>), grid, dim3(512), ctx->lds_dist, ctx->stream, (const v4i *)ctx->d_Pa,   \
+                       ctx->d_na, (const v4i *)ctx->d_Pb, ctx->d_nb, ctx->d_key, ctx->N, ctx->KS, ctx->RT, B,      \
+                       ctx->cfg.num_rot, ctx->cfg.use_flip, ctx->nrr_eff)
+    switch (ctx->NT) {
+    case 1: LAUNCH_NT(1); break;
+    case 2: LAUNCH_NT(2); break;
+    case 3: LAUNCH_NT(3); break;
+    default: LAUNCH_NT(4); break;
+    }
+#undef LAUNCH_NT
+    return launch_check(ctx, "k_dist_mfma_u8");
+}
+
 int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
+    if (ctx->mfma) {
+        TRY(run_rotpack_mfma(ctx, dev_images, B));
+        TRY(run_dist_mfma(ctx, B));
+        return PINK_HIP_OK;
+    }
     TRY(run_rotate(ctx, dev_images, B));
     TRY(run_pack_rot(ctx, B));
     TRY(run_dist(ctx, B));

@@ -87,20 +87,23 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
     if N < 331:
         som[1] = O.rotated_images(img, C_, I, D, nrot, flip)[min(3, nrot - 1)].ravel()   # an exact match
         som[2] = som[1] * np.float32(0.5)
-    with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type) as ctx:
-        ctx.set_som(som)
-        assert ctx.region_size == len(O.region(C_, D, ed, shape_))
-        d, ssd, best = ctx.distance(img)
     s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, ed_type)
     rot = O.rotated_images(img, C_, I, D, nrot, flip)
     od, ossd, obest = O.distance_matrix(s, som, rot)
-    if ed_type == capi.FLOAT:
-        # gate: 1e-5 relative, argmin identical up to ties; achieved and asserted: bit-exact
-        assert np.array_equal(bits(d), bits(od))
-    else:
-        assert np.array_equal(ssd, ossd)
-        assert np.array_equal(bits(d), bits(od))
-    assert np.array_equal(best, obest)
+    # a uint8 mapper runs on the matrix cores by default (N <= 128): check both kernels
+    choices = [capi.KERNEL_AUTO, capi.KERNEL_VALU] if ed_type == capi.UINT8 else [capi.KERNEL_AUTO]
+    for choice in choices:
+        with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type, kernel_choice=choice) as ctx:
+            ctx.set_som(som)
+            assert ctx.region_size == len(O.region(C_, D, ed, shape_))
+            d, ssd, best = ctx.distance(img)
+        if ed_type == capi.FLOAT:
+            # gate: 1e-5 relative, argmin identical up to ties; achieved and asserted: bit-exact
+            assert np.array_equal(bits(d), bits(od))
+        else:
+            assert np.array_equal(ssd, ossd), choice
+            assert np.array_equal(bits(d), bits(od)), choice
+        assert np.array_equal(best, obest), choice
 
 
 TRAIN_CASES = [
@@ -166,19 +169,22 @@ def test_reference_trainer_known_answers():
         assert bmu.tolist() == [1] and np.array_equal(ctx.get_som(), som)
 
 
-MAP_CASES = [("cfg1", 24, None), ("cfg0", 5, capi.FLOAT), ("cfg4", 300, None), ("cfg2", 2, None)]
+MAP_CASES = [("cfg1", 24, None, capi.KERNEL_AUTO), ("cfg1", 9, None, capi.KERNEL_VALU),
+             ("cfg1", 3, None, capi.KERNEL_MFMA), ("cfg0", 5, capi.FLOAT, capi.KERNEL_AUTO),
+             ("cfg4", 300, None, capi.KERNEL_AUTO), ("cfg4", 50, None, capi.KERNEL_VALU),
+             ("cfg2", 2, None, capi.KERNEL_AUTO)]
 
 
-@pytest.mark.parametrize("name,n,ed_type", MAP_CASES)
-def test_map_parity(name, n, ed_type):
+@pytest.mark.parametrize("name,n,ed_type,choice", MAP_CASES)
+def test_map_parity(name, n, ed_type, choice):
     w = synthetic.WORKLOADS[name]
     ed_type = w.ed_type if ed_type is None else ed_type
-    say("map", name, n, ed_type)
+    say("map", name, n, ed_type, choice)
     imgs = synthetic.images(w, n)
     som = synthetic.initial_som(w)
     som[3] = O.rotated_images(imgs[1], w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip)[5 % w.R].ravel()
     with capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
-                      w.ed_shape, ed_type, None, max_batch=7) as ctx:
+                      w.ed_shape, ed_type, None, max_batch=7, kernel_choice=choice) as ctx:
         ctx.set_som(som)
         heat, best = ctx.map(imgs)
     s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
@@ -225,6 +231,13 @@ def test_map_full_size_properties():
     assert np.array_equal(bits(heat2[::-1]), bits(heat)) and np.array_equal(best2[::-1], best)   # order-independent
     assert (heat >= 0).all() and np.isfinite(heat).all() and (best < w.R).all()
     assert np.array_equal(bits(heat3), bits(heat[:50]))
+
+
+def test_mfma_kernel_refused_where_it_does_not_apply():
+    with pytest.raises(capi.PinkError):
+        capi.Context(200, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.UINT8, kernel_choice=capi.KERNEL_MFMA)
+    with pytest.raises(capi.PinkError):
+        capi.Context(16, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.FLOAT, kernel_choice=capi.KERNEL_MFMA)
 
 
 def test_profiling_counts_launches():
