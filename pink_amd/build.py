@@ -35,5 +35,22 @@ def build(verbose=False, extra=()):
     return OUT
 
 
+HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_host.cpp")
+HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "test_host")
+
+
+def build_host_test(verbose=False):
+    """Compile the C++ Trainer/Mapper mirror (pink_amd/host) and its test with the host compiler."""
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-Wextra",
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "host"),
+           HOST_TEST_SRC, "-o", HOST_TEST_BIN, "-L" + os.path.join(HERE, "lib"), "-lpink_hip",
+           "-Wl,-rpath,$ORIGIN/../../pink_amd/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     build(verbose=True, extra=sys.argv[1:])
+    build_host_test(verbose=True)
