@@ -32,7 +32,7 @@
 namespace {
 
 constexpr uint32_t kWave = 64;
-constexpr uint32_t kEpadMultiple = 32;   // region length padded so k-loops need no tail
+constexpr uint32_t kEpadMultiple = 64;   // region length padded so k-loops need no tail
 constexpr int kClsRotate = 0, kClsPack = 1, kClsDist = 2, kClsUpdate = 3, kClsFinal = 4;
 
 thread_local std::string g_create_error;
@@ -285,6 +285,124 @@ __global__ __launch_bounds__(64) void k_dist_valu(const void *__restrict__ somP_
 }
 
 
+
+// ---------------------------------------------------------------------------------
+// Float32 distance + argmin: LDS-shared rotations, neuron values broadcast by DPP.
+// A block of 4 waves shares 64 consecutive rotations: their k-major rows are staged through
+// a double-buffered LDS tile (64 k x 64 rotations per stage) by coalesced 16-byte loads, so
+// every rotation element leaves L2 once per 4*TN neurons.  Wave w owns neurons
+// n0 + w*TN .. + TN, lane l owns rotation r0 + l.  Neuron values travel in VGPRs -- lane l
+// holds element k0 + 16*s + (l % 16) of slab s -- and reach all lanes of a row through the
+// DPP operand of the subtract (`v_sub_f32_dpp ... row_newbcast:k`), so a pair element costs
+// exactly one subtract and one fma and no scalar or LDS traffic for the neuron side.
+// The sum of each (neuron, rotation) pair is still one lane's sequential fma chain over k in
+// the CPU's element order (bit-faithful); only the argmin crosses lanes.
+// ---------------------------------------------------------------------------------
+constexpr uint32_t kDistKC = 64;
+
+// acc = fma(d, d, acc) with d = (element K of this lane's row of 16 lanes of a_row) - b.
+// Two instructions, kept together so the difference never outlives its use: an IEEE subtract
+// taking the neuron value through the DPP row broadcast, then a fused multiply-add.
+template <int K>
+__device__ __forceinline__ void ssd_step(float &acc, float a_row, float b)
+{
+    float d;
+    asm("v_sub_f32_dpp %1, %2, %3 row_newbcast:%4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_e32 %0, %1, %1"
+        : "+v"(acc), "=&v"(d)
+        : "v"(a_row), "v"(b), "n"(K));
+}
+
+template <int TN>
+__global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
+                                                      unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
+                                                      uint32_t R, uint32_t Rpad)
+{
+    __shared__ float4 s_rot[2][kDistKC * 16];          // [stage][k][64 rotations]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t r0 = blockIdx.x * kWave;
+    const uint32_t n0 = blockIdx.y * (4 * TN) + wave * TN;
+    const uint32_t b = blockIdx.z;
+    const float *rp = rotT + (size_t)b * Epad * Rpad + r0;
+    const float *np[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad + (lane & 15);
+    float acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
+
+    // thread t moves float4 #(t + 256*i), i < 4, of a stage: row t/16 + 16*i, column group t & 15
+    const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
+    float va[TN][4], vn[TN][4];
+    const float *lp = rp + (size_t)lrow * Rpad + lcol;
+    const size_t rstep = (size_t)16 * Rpad;
+    float4 st0 = *(const float4 *)(lp), st1 = *(const float4 *)(lp + rstep);
+    float4 st2 = *(const float4 *)(lp + 2 * rstep), st3 = *(const float4 *)(lp + 3 * rstep);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) va[j][sl] = np[j][16 * sl];
+    s_rot[0][tid] = st0;
+    s_rot[0][tid + 256] = st1;
+    s_rot[0][tid + 512] = st2;
+    s_rot[0][tid + 768] = st3;
+    __syncthreads();
+
+    const uint32_t nchunks = Epad / kDistKC;
+    for (uint32_t c = 0; c < nchunks; ++c) {
+        const uint32_t kn = (c + 1) * kDistKC;
+        if (c + 1 < nchunks) {
+            const float *ln = lp + (size_t)kn * Rpad;
+            st0 = *(const float4 *)(ln);
+            st1 = *(const float4 *)(ln + rstep);
+            st2 = *(const float4 *)(ln + 2 * rstep);
+            st3 = *(const float4 *)(ln + 3 * rstep);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) vn[j][sl] = np[j][kn + 16 * sl];
+        }
+        const float *cur = (const float *)s_rot[c & 1] + lane;
+#define PINK_STEP(SL, K)                                                        \
+    {                                                                           \
+        const float bv = cur[((SL) * 16 + (K)) * 64];                           \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j) ssd_step<K>(acc[j], va[j][SL], bv); \
+    }
+#define PINK_SLAB(SL)                                                                                     \
+    PINK_STEP(SL, 0) PINK_STEP(SL, 1) PINK_STEP(SL, 2) PINK_STEP(SL, 3) PINK_STEP(SL, 4) PINK_STEP(SL, 5)   \
+    PINK_STEP(SL, 6) PINK_STEP(SL, 7) PINK_STEP(SL, 8) PINK_STEP(SL, 9) PINK_STEP(SL, 10) PINK_STEP(SL, 11) \
+    PINK_STEP(SL, 12) PINK_STEP(SL, 13) PINK_STEP(SL, 14) PINK_STEP(SL, 15)
+        // (a VALU write of a DPP source needs two idle slots before the DPP read: the copies
+        // of the prefetched neuron values at the end of the previous pass are far away, the
+        // no-op makes that independent of what the compiler schedules next to this point)
+        asm volatile("s_nop 1");
+        PINK_SLAB(0) PINK_SLAB(1) PINK_SLAB(2) PINK_SLAB(3)
+#undef PINK_SLAB
+#undef PINK_STEP
+        if (c + 1 < nchunks) {
+            float4 *nx = s_rot[(c + 1) & 1];
+            nx[tid] = st0;
+            nx[tid + 256] = st1;
+            nx[tid + 512] = st2;
+            nx[tid + 768] = st3;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int sl = 0; sl < 4; ++sl) va[j][sl] = vn[j][sl];
+        }
+        __syncthreads();
+    }
+
+    const uint32_t r = r0 + lane;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | r;
+        if (r >= R) kv = ~0ull;
+        kv = wave_min_u64(kv);
+        if (lane == 0 && n0 + j < N) atomicMin(&key[(size_t)b * N + n0 + j], kv);
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // uint8 distance on the matrix cores (mapping).
 //
@@ -489,12 +607,15 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
 // BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
 // Every block recomputes the best-matching neuron from the N keys (first minimum wins),
 // then block (part, n) pulls its slice of neuron n toward that neuron's best variant:
-//   w = w - ((w - x) * f),  f = factors[bmu * N + n], skipped when f == 0.
+//   w = w - ((w - x) * f),  f = factors[bmu * N + n], skipped when f == 0,
+// and refreshes the region elements of the packed distance operand in the same pass.
 // ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const float *__restrict__ rot,
                                                 const unsigned long long *__restrict__ key,
                                                 const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
-                                                uint32_t N, uint32_t S, uint32_t parts, uint32_t shift)
+                                                uint32_t N, uint32_t S, uint32_t parts, uint32_t shift,
+                                                void *__restrict__ somP, const uint32_t *__restrict__ inv,
+                                                uint32_t Epad, float qfactor)
 {
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
@@ -529,7 +650,17 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
     for (uint32_t j = j0 + tid; j < j1; j += 256) {
         const float wv = w[j];
-        w[j] = __fsub_rn(wv, __fmul_rn(__fsub_rn(wv, x[j]), f));
+        const float nv = __fsub_rn(wv, __fmul_rn(__fsub_rn(wv, x[j]), f));
+        w[j] = nv;
+        // keep the distance kernel's packed copy of the region current (inv = position of element
+        // j in the region, or none)
+        if (inv) {
+            const uint32_t k = inv[j];
+            if (k != 0xffffffffu) {
+                if (qfactor > 0.0f) ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
+                else ((float *)somP)[(size_t)n * Epad + k] = nv;
+            }
+        }
     }
 }
 
@@ -582,6 +713,7 @@ struct pink_hip_ctx {
     unsigned long long *d_key = nullptr;
     void *d_somP = nullptr, *d_rotT = nullptr;
     uint32_t *d_bmu_scratch = nullptr;
+    uint32_t *d_inv = nullptr;   // element of a neuron -> position in the region (none: ~0); null if not one-to-one
     float *d_dist = nullptr;
     long long *d_ssd = nullptr;
     uint32_t *d_best = nullptr;
@@ -760,7 +892,7 @@ int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 }
 
 template <int MODE>
-void launch_dist(pink_hip_ctx *ctx, uint32_t B)
+void launch_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     // Neurons per wave: as many as keep at least ~2 waves per SIMD in flight.
     const uint32_t rblocks = ctx->Rpad / kWave;
@@ -768,8 +900,10 @@ void launch_dist(pink_hip_ctx *ctx, uint32_t B)
     uint32_t tn = 8;
     while (tn > 1 && (size_t)rblocks * ((ctx->N + tn - 1) / tn) * B < target_waves) tn >>= 1;
     const dim3 grid(rblocks, (ctx->N + tn - 1) / tn, B);
+    const void *rotT = (const char *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad * 4;
+    unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
 #define LAUNCH_TN(T_)                                                                                           \
-    hipLaunchKernelGGL((k_dist_valu<MODE, T_>), grid, dim3(64), 0, ctx->stream, ctx->d_somP, ctx->d_rotT, ctx->d_key, \
+    hipLaunchKernelGGL((k_dist_valu<MODE, T_>), grid, dim3(64), 0, ctx->stream, ctx->d_somP, rotT, key,        \
                        ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
     switch (tn) {
     case 8: LAUNCH_TN(8); break;
@@ -780,24 +914,52 @@ void launch_dist(pink_hip_ctx *ctx, uint32_t B)
 #undef LAUNCH_TN
 }
 
-int run_dist(pink_hip_ctx *ctx, uint32_t B)
+// Distance + argmin of B images starting at image slot `slot` of the current launch group.
+void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
+{
+    // Neurons per block = 4 waves x TN: the largest TN that still leaves about four waves per SIMD
+    // (TN = 1 spends as long in LDS reads as in arithmetic, so it is the last resort).
+    const uint32_t rblocks = ctx->Rpad / kWave;
+    uint32_t tn = 8;
+    while (tn > 1 && (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B < (size_t)4 * ctx->num_cu) tn >>= 1;
+    const dim3 grid(rblocks, (ctx->N + 4 * tn - 1) / (4 * tn), B);
+    const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
+    unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
+#define LAUNCH_TN(T_)                                                                                              \
+    hipLaunchKernelGGL((k_dist_f32_dpp<T_>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
+                       ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    switch (tn) {
+    case 8: LAUNCH_TN(8); break;
+    case 4: LAUNCH_TN(4); break;
+    case 2: LAUNCH_TN(2); break;
+    default: LAUNCH_TN(1); break;
+    }
+#undef LAUNCH_TN
+}
+
+int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     Timed t(ctx, kClsDist);
     switch (ctx->cfg.ed_type) {
-    case PINK_HIP_FLOAT: launch_dist<0>(ctx, B); break;
-    case PINK_HIP_UINT8: launch_dist<1>(ctx, B); break;
-    default: launch_dist<2>(ctx, B); break;
+    case PINK_HIP_FLOAT:
+        if (ctx->cfg.kernel_choice == PINK_HIP_KERNEL_VALU) launch_dist<0>(ctx, slot, B);   // one wave per block, no LDS
+        else launch_dist_f32(ctx, slot, B);
+        break;
+    case PINK_HIP_UINT8: launch_dist<1>(ctx, slot, B); break;
+    default: launch_dist<2>(ctx, slot, B); break;
     }
     return launch_check(ctx, "k_dist");
 }
 
-int run_update(pink_hip_ctx *ctx, uint32_t *dev_bmu_out)
+int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
 {
     Timed t(ctx, kClsUpdate);
     uint32_t parts = (1024 + ctx->N - 1) / ctx->N;
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
-    hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_rot, ctx->d_key,
-                       ctx->d_factors, dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift);
+    hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
+                       ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
+                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP, ctx->d_inv, ctx->Epad,
+                       is_int(ctx) ? (float)ctx->factor : 0.0f);
     return launch_check(ctx, "k_update");
 }
 
@@ -819,7 +981,7 @@ int free_all(pink_hip_ctx *ctx)
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
-                    ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need};
+                    ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -917,8 +1079,13 @@ int init_ctx(pink_hip_ctx *ctx)
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
     size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
     if (ctx->mfma) per_image = (size_t)ctx->RT * ctx->KS * 1024 + (size_t)ctx->RT * 128 + (size_t)ctx->N * 24;
-    if (ctx->trainer) ctx->Bcap = 1;
-    else {
+    if (ctx->trainer) {
+        // images whose variants are prepared ahead of the sequential distance/update chain
+        size_t b = c.max_batch ? c.max_batch : 64;
+        const size_t budget = (size_t)2 << 30;
+        while (b > 1 && b * per_image > budget) b >>= 1;
+        ctx->Bcap = (uint32_t)b;
+    } else {
         size_t b = c.max_batch ? c.max_batch : (ctx->mfma ? 2048 : 256);
         const size_t budget = (size_t)4 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
@@ -947,6 +1114,17 @@ int init_ctx(pink_hip_ctx *ctx)
     TRY(dev_alloc(ctx, &ctx->d_ssd, B * ctx->N));
     TRY(dev_alloc(ctx, &ctx->d_best, B * ctx->N));
     if (ctx->trainer) {
+        // element -> region position, when every region element is a distinct neuron element
+        std::vector<uint32_t> inv(ctx->S, 0xffffffffu);
+        bool one_to_one = true;
+        for (uint32_t k = 0; k < ctx->E; ++k) {
+            if (inv[region[k]] != 0xffffffffu) one_to_one = false;
+            inv[region[k]] = k;
+        }
+        if (one_to_one) {
+            TRY(dev_alloc(ctx, &ctx->d_inv, inv.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_inv, inv.data(), inv.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        }
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
@@ -995,7 +1173,7 @@ int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
     }
     TRY(run_rotate(ctx, dev_images, B));
     TRY(run_pack_rot(ctx, B));
-    TRY(run_dist(ctx, B));
+    TRY(run_dist(ctx, 0, B));
     return PINK_HIP_OK;
 }
 
@@ -1100,10 +1278,17 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
     if (!ctx || (!dev_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train_device: null argument");
     if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_train: context was created without update factors");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    for (uint32_t i = 0; i < n_images; ++i) {
-        TRY(distance_group(ctx, dev_images + (size_t)i * ctx->isz, 1));
-        TRY(run_update(ctx, dev_bmu_out ? dev_bmu_out + i : ctx->d_bmu_scratch));
-        TRY(run_pack_som(ctx));
+    // The variants of an image and their packed distance operand do not depend on the SOM: they
+    // are produced for a group of images per launch.  Distance and update stay strictly sequential.
+    for (uint32_t done = 0; done < n_images; done += ctx->Bcap) {
+        const uint32_t B = std::min(ctx->Bcap, n_images - done);
+        TRY(run_rotate(ctx, dev_images + (size_t)done * ctx->isz, B));
+        TRY(run_pack_rot(ctx, B));
+        for (uint32_t b = 0; b < B; ++b) {
+            TRY(run_dist(ctx, b, 1));
+            TRY(run_update(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
+            if (!ctx->d_inv) TRY(run_pack_som(ctx));
+        }
     }
     return PINK_HIP_OK;
 }
