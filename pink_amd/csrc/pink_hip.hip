@@ -21,6 +21,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -220,6 +221,20 @@ __global__ __launch_bounds__(256) void k_pack_rot(const float *__restrict__ rot,
     }
 }
 
+// Float32 operand of the DPP distance kernel: rotP[b][r][k] = rot[b][r][off[k]], the region of
+// every variant contiguous in k (rows r >= R and elements k >= E are zero).
+__global__ __launch_bounds__(256) void k_pack_rot_rows(const float *__restrict__ rot, const uint32_t *__restrict__ off,
+                                                       float *__restrict__ rotP, uint32_t R, uint32_t S, uint32_t E,
+                                                       uint32_t Epad, uint32_t Rpad)
+{
+    const uint32_t b = blockIdx.z, r = blockIdx.y;
+    const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= Epad) return;
+    float v = 0.0f;
+    if (r < R && k < E) v = rot[((size_t)b * R + r) * S + off[k]];
+    rotP[((size_t)b * Rpad + r) * Epad + k] = v;
+}
+
 // ---------------------------------------------------------------------------------
 // Distance + argmin over rotations on the vector ALU.
 // One wave = 64 consecutive rotations x TN neurons.  Lane l owns rotation r0 + l and TN
@@ -288,42 +303,39 @@ __global__ __launch_bounds__(64) void k_dist_valu(const void *__restrict__ somP_
 
 // ---------------------------------------------------------------------------------
 // Float32 distance + argmin: LDS-shared rotations, neuron values broadcast by DPP.
-// A block of 4 waves shares 64 consecutive rotations: their k-major rows are staged through
-// a double-buffered LDS tile (64 k x 64 rotations per stage) by coalesced 16-byte loads, so
-// every rotation element leaves L2 once per 4*TN neurons.  Wave w owns neurons
-// n0 + w*TN .. + TN, lane l owns rotation r0 + l.  Neuron values travel in VGPRs -- lane l
-// holds element k0 + 16*s + (l % 16) of slab s -- and reach all lanes of a row through the
-// DPP operand of the subtract (`v_sub_f32_dpp ... row_newbcast:k`), so a pair element costs
-// exactly one subtract and one fma and no scalar or LDS traffic for the neuron side.
+// A block of 4 waves shares 64 consecutive rotations.  Their packed regions (k contiguous per
+// rotation) are staged through a double-buffered LDS tile of 64 rotations x 64 elements by
+// coalesced 16-byte loads, so every rotation element leaves L2 once per 4*TN neurons; a lane
+// reads its own rotation's row back 16 bytes at a time (row stride 68 words: conflict-free).
+// Wave w owns neurons n0 + w*TN .. + TN, lane l owns rotation r0 + l.  Neuron values travel in
+// VGPRs -- lane l holds element k0 + 16*s + (l % 16) of slab s -- and reach all lanes of a row
+// through the DPP operand of the subtract (`v_sub_f32_dpp ... row_newbcast:k`), so a pair
+// element costs exactly one subtract and one fma and no scalar or LDS traffic for the neuron side.
 // The sum of each (neuron, rotation) pair is still one lane's sequential fma chain over k in
 // the CPU's element order (bit-faithful); only the argmin crosses lanes.
 // ---------------------------------------------------------------------------------
 constexpr uint32_t kDistKC = 64;
+constexpr uint32_t kDistRow = kDistKC + 4;   // LDS row stride in floats
 
-// acc = fma(d, d, acc) with d = (element K of this lane's row of 16 lanes of a_row) - b.
-// Two instructions, kept together so the difference never outlives its use: an IEEE subtract
-// taking the neuron value through the DPP row broadcast, then a fused multiply-add.
-template <int K>
-__device__ __forceinline__ void ssd_step(float &acc, float a_row, float b)
-{
-    float d;
-    asm("v_sub_f32_dpp %1, %2, %3 row_newbcast:%4 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_e32 %0, %1, %1"
-        : "+v"(acc), "=&v"(d)
-        : "v"(a_row), "v"(b), "n"(K));
-}
+// The inner blocks (inline assembly: DPP subtracts issued ahead of the multiply-adds that use
+// them) are generated by gen_ssd_steps.py.
+#include "ssd_steps.inc"
 
-template <int TN>
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// HB = rotation values fetched from LDS per batch (64: a whole stage at once, for small TN where a
+// wave has little else to overlap the LDS latency with; 16 otherwise).
+template <int TN, int PD, int HB>
 __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
-                                                      unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
-                                                      uint32_t R, uint32_t Rpad)
+                                                         unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
+                                                         uint32_t R, uint32_t Rpad)
 {
-    __shared__ float4 s_rot[2][kDistKC * 16];          // [stage][k][64 rotations]
+    __shared__ v4f s_rot[2][64 * kDistRow / 4];          // [stage][64 rotations][64 elements + 4]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r0 = blockIdx.x * kWave;
     const uint32_t n0 = blockIdx.y * (4 * TN) + wave * TN;
     const uint32_t b = blockIdx.z;
-    const float *rp = rotT + (size_t)b * Epad * Rpad + r0;
+    const float *rp = rotT + ((size_t)b * Rpad + r0) * Epad;
     const float *np[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad + (lane & 15);
@@ -331,67 +343,104 @@ __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
 
-    // thread t moves float4 #(t + 256*i), i < 4, of a stage: row t/16 + 16*i, column group t & 15
+    // Thread t moves 4 vectors of a stage: rotation t/16 + 16*i (i < 4), elements 4*(t & 15) .. +4.
+    // Chunks c+1 .. c+PD are in flight in registers while chunk c is computed from LDS.
     const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
-    float va[TN][4], vn[TN][4];
-    const float *lp = rp + (size_t)lrow * Rpad + lcol;
-    const size_t rstep = (size_t)16 * Rpad;
-    float4 st0 = *(const float4 *)(lp), st1 = *(const float4 *)(lp + rstep);
-    float4 st2 = *(const float4 *)(lp + 2 * rstep), st3 = *(const float4 *)(lp + 3 * rstep);
+    const float *lp = rp + (size_t)lrow * Epad + lcol;
+    const size_t rstep = (size_t)16 * Epad;
+    const uint32_t lds_w = (lrow * kDistRow + lcol) / 4;      // vector index of this thread's first store
+    const uint32_t lds_wstep = 16 * kDistRow / 4;
+    const uint32_t nchunks = Epad / kDistKC;
+    v4f st[PD][4];
+    float vn[PD][4][TN];     // [slot][slab][neuron]: lane l holds element 16*slab + l%16 of the chunk
+    float va[4][TN];
+
+    {
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < 4; ++i) s_rot[0][lds_w + i * lds_wstep] = *(const v4f *)(lp + i * rstep);
 #pragma unroll
-        for (int sl = 0; sl < 4; ++sl) va[j][sl] = np[j][16 * sl];
-    s_rot[0][tid] = st0;
-    s_rot[0][tid + 256] = st1;
-    s_rot[0][tid + 512] = st2;
-    s_rot[0][tid + 768] = st3;
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) va[sl][j] = np[j][16 * sl];
+#pragma unroll
+        for (int u = 0; u < PD; ++u) {
+            if (u + 1 < nchunks) {
+                const uint32_t k = (u + 1) * kDistKC;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) st[u][i] = *(const v4f *)(lp + k + i * rstep);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int sl = 0; sl < 4; ++sl) vn[u][sl][j] = np[j][k + 16 * sl];
+            }
+        }
+    }
     __syncthreads();
 
-    const uint32_t nchunks = Epad / kDistKC;
-    for (uint32_t c = 0; c < nchunks; ++c) {
-        const uint32_t kn = (c + 1) * kDistKC;
-        if (c + 1 < nchunks) {
-            const float *ln = lp + (size_t)kn * Rpad;
-            st0 = *(const float4 *)(ln);
-            st1 = *(const float4 *)(ln + rstep);
-            st2 = *(const float4 *)(ln + 2 * rstep);
-            st3 = *(const float4 *)(ln + 3 * rstep);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int sl = 0; sl < 4; ++sl) vn[j][sl] = np[j][kn + 16 * sl];
-        }
-        const float *cur = (const float *)s_rot[c & 1] + lane;
-#define PINK_STEP(SL, K)                                                        \
-    {                                                                           \
-        const float bv = cur[((SL) * 16 + (K)) * 64];                           \
-        _Pragma("unroll") for (int j = 0; j < TN; ++j) ssd_step<K>(acc[j], va[j][SL], bv); \
+#define PINK_SLAB(SL)                                                                                      \
+    {                                                                                                      \
+        if (HB == 16 || (SL) == 0) {                                                                       \
+            /* fetch the next HB elements of this lane's rotation from LDS in one batch, then compute */  \
+            _Pragma("unroll") for (int q = 0; q < HB / 4; ++q) {                                           \
+                const v4f t4 = cur[(SL) * 4 + q];                                                          \
+                bv[4 * q] = t4.x; bv[4 * q + 1] = t4.y; bv[4 * q + 2] = t4.z; bv[4 * q + 3] = t4.w;        \
+            }                                                                                              \
+            __builtin_amdgcn_sched_barrier(0);                                                             \
+        }                                                                                                  \
+        const float *bs = bv + ((SL) * 16) % HB;                                                           \
+        if constexpr (TN == 1) {                                                                           \
+            ssd_block<0>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs);                                  \
+        } else if constexpr (TN == 2) {                                                                    \
+            ssd_block<0>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs);                                  \
+            ssd_block<8>(acc, va[SL], bs); ssd_block<12>(acc, va[SL], bs);                                 \
+        } else if constexpr (TN == 4) {                                                                    \
+            ssd_block<0>(acc, va[SL], bs); ssd_block<2>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs);   \
+            ssd_block<6>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs); ssd_block<10>(acc, va[SL], bs);  \
+            ssd_block<12>(acc, va[SL], bs); ssd_block<14>(acc, va[SL], bs);                                \
+        } else {                                                                                           \
+            ssd_block<0>(acc, va[SL], bs); ssd_block<1>(acc, va[SL], bs); ssd_block<2>(acc, va[SL], bs);   \
+            ssd_block<3>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs); ssd_block<5>(acc, va[SL], bs);   \
+            ssd_block<6>(acc, va[SL], bs); ssd_block<7>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs);   \
+            ssd_block<9>(acc, va[SL], bs); ssd_block<10>(acc, va[SL], bs); ssd_block<11>(acc, va[SL], bs); \
+            ssd_block<12>(acc, va[SL], bs); ssd_block<13>(acc, va[SL], bs); ssd_block<14>(acc, va[SL], bs);\
+            ssd_block<15>(acc, va[SL], bs);                                                                \
+        }                                                                                                  \
     }
-#define PINK_SLAB(SL)                                                                                     \
-    PINK_STEP(SL, 0) PINK_STEP(SL, 1) PINK_STEP(SL, 2) PINK_STEP(SL, 3) PINK_STEP(SL, 4) PINK_STEP(SL, 5)   \
-    PINK_STEP(SL, 6) PINK_STEP(SL, 7) PINK_STEP(SL, 8) PINK_STEP(SL, 9) PINK_STEP(SL, 10) PINK_STEP(SL, 11) \
-    PINK_STEP(SL, 12) PINK_STEP(SL, 13) PINK_STEP(SL, 14) PINK_STEP(SL, 15)
-        // (a VALU write of a DPP source needs two idle slots before the DPP read: the copies
-        // of the prefetched neuron values at the end of the previous pass are far away, the
-        // no-op makes that independent of what the compiler schedules next to this point)
-        asm volatile("s_nop 1");
-        PINK_SLAB(0) PINK_SLAB(1) PINK_SLAB(2) PINK_SLAB(3)
+
+    for (uint32_t c0 = 0; c0 < nchunks; c0 += PD) {
+#pragma unroll
+        for (int u = 0; u < PD; ++u) {
+            const uint32_t c = c0 + u;          // chunk c+1 waits in register slot u
+            if (c < nchunks) {
+                const v4f *cur = s_rot[c & 1] + lane * (kDistRow / 4);
+                float bv[HB];
+                // (a VALU write of a DPP source needs two idle slots before the DPP read; the no-op
+                // makes that independent of what the compiler schedules next to this point)
+                asm volatile("s_nop 1");
+                PINK_SLAB(0) PINK_SLAB(1) PINK_SLAB(2) PINK_SLAB(3)
+                if (c + 1 < nchunks) {
+                    v4f *nx = s_rot[(c + 1) & 1];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) nx[lds_w + i * lds_wstep] = st[u][i];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int sl = 0; sl < 4; ++sl) va[sl][j] = vn[u][sl][j];
+                }
+                if (c + 1 + PD < nchunks) {
+                    const uint32_t k = (c + 1 + PD) * kDistKC;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) st[u][i] = *(const v4f *)(lp + k + i * rstep);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int sl = 0; sl < 4; ++sl) vn[u][sl][j] = np[j][k + 16 * sl];
+                }
+                __syncthreads();
+            }
+        }
+    }
 #undef PINK_SLAB
-#undef PINK_STEP
-        if (c + 1 < nchunks) {
-            float4 *nx = s_rot[(c + 1) & 1];
-            nx[tid] = st0;
-            nx[tid + 256] = st1;
-            nx[tid + 512] = st2;
-            nx[tid + 768] = st3;
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int sl = 0; sl < 4; ++sl) va[j][sl] = vn[j][sl];
-        }
-        __syncthreads();
-    }
 
     const uint32_t r = r0 + lane;
 #pragma unroll
@@ -728,6 +777,8 @@ struct pink_hip_ctx {
     unsigned short *d_poff = nullptr;
     uint32_t *d_need = nullptr;
 
+    uint32_t force_tn = 0;     // tuning aid: PINK_HIP_DIST_TN=1|2|4|8 overrides the neurons-per-wave choice
+
     bool profiling = false;
     std::vector<EventPair> events;
     std::vector<hipEvent_t> event_pool;
@@ -881,6 +932,11 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 {
     Timed t(ctx, kClsPack);
+    if (!is_int(ctx)) {
+        hipLaunchKernelGGL(k_pack_rot_rows, dim3((ctx->Epad + 255) / 256, ctx->Rpad, B), dim3(256), 0, ctx->stream,
+                           ctx->d_rot, ctx->d_region, (float *)ctx->d_rotT, ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad);
+        return launch_check(ctx, "k_pack_rot_rows");
+    }
     const dim3 grid(ctx->Epad / 32, ctx->Rpad / 32, B);
     if (is_int(ctx))
         hipLaunchKernelGGL(k_pack_rot<true>, grid, dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region, ctx->d_rotT,
@@ -920,19 +976,20 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     // Neurons per block = 4 waves x TN: the largest TN that still leaves about four waves per SIMD
     // (TN = 1 spends as long in LDS reads as in arithmetic, so it is the last resort).
     const uint32_t rblocks = ctx->Rpad / kWave;
-    uint32_t tn = 8;
+    uint32_t tn = 4;
     while (tn > 1 && (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B < (size_t)4 * ctx->num_cu) tn >>= 1;
+    if (ctx->force_tn) tn = std::min(ctx->force_tn, 4u);
     const dim3 grid(rblocks, (ctx->N + 4 * tn - 1) / (4 * tn), B);
     const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
-#define LAUNCH_TN(T_)                                                                                              \
-    hipLaunchKernelGGL((k_dist_f32_dpp<T_>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
+#define LAUNCH_TN(...)                                                                                             \
+    hipLaunchKernelGGL((k_dist_f32_dpp<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
                        ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    // second parameter: chunks of operand prefetch held in registers (deep where waves are few)
     switch (tn) {
-    case 8: LAUNCH_TN(8); break;
-    case 4: LAUNCH_TN(4); break;
-    case 2: LAUNCH_TN(2); break;
-    default: LAUNCH_TN(1); break;
+    case 4: LAUNCH_TN(4, 2, 16); break;
+    case 2: LAUNCH_TN(2, 1, 64); break;
+    default: LAUNCH_TN(1, 2, 64); break;
     }
 #undef LAUNCH_TN
 }
@@ -941,10 +998,7 @@ int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     Timed t(ctx, kClsDist);
     switch (ctx->cfg.ed_type) {
-    case PINK_HIP_FLOAT:
-        if (ctx->cfg.kernel_choice == PINK_HIP_KERNEL_VALU) launch_dist<0>(ctx, slot, B);   // one wave per block, no LDS
-        else launch_dist_f32(ctx, slot, B);
-        break;
+    case PINK_HIP_FLOAT: launch_dist_f32(ctx, slot, B); break;
     case PINK_HIP_UINT8: launch_dist<1>(ctx, slot, B); break;
     default: launch_dist<2>(ctx, slot, B); break;
     }
@@ -1224,6 +1278,10 @@ int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
     ctx->device = cfg->device;
     ctx->factor = cfg->ed_type == PINK_HIP_UINT8 ? 255u : cfg->ed_type == PINK_HIP_UINT16 ? 65535u : 1u;
     ctx->shift = cfg->ed_type == PINK_HIP_FLOAT ? 32u : 16u;
+    if (const char *e = getenv("PINK_HIP_DIST_TN")) {
+        const int v = atoi(e);
+        if (v == 1 || v == 2 || v == 4 || v == 8) ctx->force_tn = (uint32_t)v;
+    }
 
     int rc = init_ctx(ctx);
     if (rc != PINK_HIP_OK) {
