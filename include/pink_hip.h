@@ -60,9 +60,10 @@ typedef enum { PINK_HIP_STEP = 0, PINK_HIP_GAUSSIAN = 1, PINK_HIP_UNITY_GAUSSIAN
 
 /* Which distance kernel a context uses (debugging / measurement knob). */
 typedef enum {
-    PINK_HIP_KERNEL_AUTO = 0,   /* float32: sequential-FMA VALU kernel; integer modes: int8 MFMA */
-    PINK_HIP_KERNEL_VALU = 1,   /* integer modes on the vector ALU in exact int32/int64          */
-    PINK_HIP_KERNEL_MFMA = 2
+    PINK_HIP_KERNEL_AUTO = 0,      /* float32: sequential-fma vector-ALU kernel; uint8 mapper: int8 MFMA where it applies */
+    PINK_HIP_KERNEL_VALU = 1,      /* integer modes on the vector ALU in exact int32/int64                */
+    PINK_HIP_KERNEL_MFMA = 2,      /* uint8 mapper, int8 MFMA, symmetries applied to the image variants   */
+    PINK_HIP_KERNEL_MFMA_SYM = 3   /* uint8 mapper, int8 MFMA, symmetries applied to the SOM once         */
 } pink_hip_kernel_choice;
 
 /*

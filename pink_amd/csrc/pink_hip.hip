@@ -652,6 +652,8 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
     }
 }
 
+#include "mfma_u8_sym.inc"
+
 // ---------------------------------------------------------------------------------
 // BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
 // Every block recomputes the best-matching neuron from the N keys (first minimum wins),
@@ -776,6 +778,11 @@ struct pink_hip_ctx {
     int *d_na = nullptr, *d_nb = nullptr;
     unsigned short *d_poff = nullptr;
     uint32_t *d_need = nullptr;
+    // uint8 mapping with the symmetries on the SOM side
+    bool mfma_sym = false;
+    uint32_t Ku = 0, KSs = 0, RTP = 0, slices = 0, groups = 1, all_sym = 0;
+    uint32_t *d_upos = nullptr, *d_aoff = nullptr;
+    unsigned char *d_kmask = nullptr;
 
     uint32_t force_tn = 0;     // tuning aid: PINK_HIP_DIST_TN=1|2|4|8 overrides the neurons-per-wave choice
 
@@ -902,6 +909,11 @@ bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT
 int run_pack_som(pink_hip_ctx *ctx)
 {
     Timed t(ctx, kClsPack);
+    if (ctx->mfma_sym) {
+        hipLaunchKernelGGL(k_pack_som_sym_u8, dim3(ctx->slices * 8 * 32), dim3(256), 0, ctx->stream, ctx->d_som,
+                           ctx->d_aoff, ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->KSs);
+        return launch_check(ctx, "k_pack_som_sym_u8");
+    }
     if (ctx->mfma) {
         hipLaunchKernelGGL(k_pack_som_u8, dim3(ctx->NT * 32), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
                            ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->E, ctx->KS);
@@ -1035,7 +1047,8 @@ int free_all(pink_hip_ctx *ctx)
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
-                    ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv};
+                    ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -1092,7 +1105,87 @@ int init_ctx(pink_hip_ctx *ctx)
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA && !fits)
             return fail(ctx, PINK_HIP_EINVAL, "the MFMA distance kernel needs a uint8 mapper with at most 128 neurons "
                                               "whose packed SOM fits in LDS");
-        ctx->mfma = fits && c.kernel_choice != PINK_HIP_KERNEL_VALU;
+        ctx->mfma = fits && (c.kernel_choice == PINK_HIP_KERNEL_AUTO || c.kernel_choice == PINK_HIP_KERNEL_MFMA);
+    }
+    // Symmetries on the SOM side: needs the union of the symmetric images of the region to fit 32
+    // k-steps held in registers and at most 96 base rotations per image.
+    {
+        const uint32_t D = ctx->D, DD = D * D;
+        std::vector<std::vector<uint32_t>> pos(8);      // pos[sym][e] = perm_sym(region[e])
+        std::vector<char> in_union(ctx->S, 0);
+        std::vector<bool> sym_valid(8);
+        for (uint32_t sym = 0; sym < 8; ++sym) {
+            const uint32_t f = sym >> 2, q = sym & 3;
+            sym_valid[sym] = (c.num_rot != 1 || q == 0) && (c.use_flip || f == 0);
+            pos[sym].resize(ctx->E);
+            for (uint32_t e = 0; e < ctx->E; ++e) {
+                const uint32_t ch = region[e] / DD, x = (region[e] % DD) / D, y = region[e] % D;
+                const uint32_t xs = f ? D - 1 - x : x;
+                uint32_t a, bb;
+                switch (q) {
+                case 0: a = xs; bb = y; break;
+                case 1: a = D - 1 - y; bb = xs; break;
+                case 2: a = D - 1 - xs; bb = D - 1 - y; break;
+                default: a = y; bb = D - 1 - xs; break;
+                }
+                pos[sym][e] = ch * DD + a * D + bb;
+                if (sym_valid[sym]) in_union[pos[sym][e]] = 1;
+            }
+        }
+        std::vector<uint32_t> upos;
+        std::vector<uint32_t> index_of(ctx->S, 0xffffffffu);
+        for (uint32_t p = 0; p < ctx->S; ++p)     // packed as channel << 24 | x << 12 | y
+            if (in_union[p]) {
+                index_of[p] = (uint32_t)upos.size();
+                upos.push_back(((p / DD) << 24) | (((p % DD) / D) << 12) | (p % D));
+            }
+        ctx->Ku = (uint32_t)upos.size();
+        const uint32_t ks_need = (ctx->Ku + 31) / 32;
+        ctx->KSs = ks_need <= 8 ? 8 : ks_need <= 16 ? 16 : ks_need <= 24 ? 24 : 32;
+        ctx->RTP = (ctx->nrr_eff + 31) / 32;
+        const uint32_t col_tiles = (8 * ctx->N + 31) / 32;
+        ctx->slices = (col_tiles + 7) / 8;                 // 4 waves x 2 column tiles per block
+        ctx->groups = std::max(1u, (uint32_t)ctx->num_cu / ctx->slices);
+        // a region element must not repeat (the multi-channel circular rule repeats channel 0)
+        bool distinct = true;
+        {
+            std::vector<char> seen(ctx->S, 0);
+            for (uint32_t e = 0; e < ctx->E; ++e) { if (seen[region[e]]) distinct = false; seen[region[e]] = 1; }
+        }
+        const size_t lds_img = (size_t)ctx->C * (ctx->I + 1) * (ctx->I + 1) * sizeof(float);
+        const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 32 && ctx->RTP <= 3 &&
+                              lds_img <= 150 * 1024 && D < 4096 && ctx->C < 256;
+        if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM && !fits_sym)
+            return fail(ctx, PINK_HIP_EINVAL, "the symmetric MFMA distance kernel needs a uint8 mapper, at most 1024 "
+                                              "region elements (union over the symmetries) and at most 384 rotations");
+        ctx->mfma_sym = fits_sym && (c.kernel_choice == PINK_HIP_KERNEL_AUTO || c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM);
+        if (ctx->mfma_sym) {
+            ctx->mfma = false;
+            const uint32_t Kp = ctx->KSs * 32;
+            std::vector<uint32_t> aoff((size_t)8 * Kp, 0xffffffffu);
+            std::vector<unsigned char> kmask(Kp, 0);
+            for (uint32_t sym = 0; sym < 8; ++sym) {
+                if (!sym_valid[sym]) continue;
+                for (uint32_t e = 0; e < ctx->E; ++e) {
+                    const uint32_t k = index_of[pos[sym][e]];
+                    aoff[(size_t)sym * Kp + k] = region[e];
+                    kmask[k] |= (unsigned char)(1u << sym);
+                }
+            }
+            // all valid symmetries cover the whole union: one norm per base rotation serves them all
+            unsigned char valid_bits = 0;
+            for (uint32_t sym = 0; sym < 8; ++sym) if (sym_valid[sym]) valid_bits |= (unsigned char)(1u << sym);
+            ctx->all_sym = 1;
+            for (uint32_t k = 0; k < ctx->Ku; ++k) if ((kmask[k] & valid_bits) != valid_bits) ctx->all_sym = 0;
+            TRY(dev_alloc(ctx, &ctx->d_upos, upos.size()));
+            TRY(dev_alloc(ctx, &ctx->d_aoff, aoff.size()));
+            TRY(dev_alloc(ctx, &ctx->d_kmask, kmask.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_upos, upos.data(), upos.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_aoff, aoff.data(), aoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_kmask, kmask.data(), kmask.size(), hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotpack_sym_u8, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)lds_img));
+        }
     }
     if (ctx->mfma) {
         // poff[sym][e]: where region element e of symmetry sym = flip*4 + quarter sits in the base rotation.
@@ -1133,6 +1226,7 @@ int init_ctx(pink_hip_ctx *ctx)
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
     size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
     if (ctx->mfma) per_image = (size_t)ctx->RT * ctx->KS * 1024 + (size_t)ctx->RT * 128 + (size_t)ctx->N * 24;
+    if (ctx->mfma_sym) per_image = (size_t)ctx->RTP * ctx->KSs * 1024 + (size_t)ctx->RTP * 32 * 8 * 4 + (size_t)ctx->N * 24;
     if (ctx->trainer) {
         // images whose variants are prepared ahead of the sequential distance/update chain
         size_t b = c.max_batch ? c.max_batch : 64;
@@ -1140,7 +1234,7 @@ int init_ctx(pink_hip_ctx *ctx)
         while (b > 1 && b * per_image > budget) b >>= 1;
         ctx->Bcap = (uint32_t)b;
     } else {
-        size_t b = c.max_batch ? c.max_batch : (ctx->mfma ? 2048 : 256);
+        size_t b = c.max_batch ? c.max_batch : ((ctx->mfma || ctx->mfma_sym) ? 2048 : 256);
         const size_t budget = (size_t)4 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
         ctx->Bcap = (uint32_t)b;
@@ -1152,9 +1246,14 @@ int init_ctx(pink_hip_ctx *ctx)
     HIP_TRY(ctx, hipMemset(ctx->d_som, 0, (size_t)ctx->N * ctx->S * sizeof(float)));
     // The float variants are only materialised per launch group on the vector-ALU path; the
     // matrix-core path keeps room for one image (pink_hip_rotate).
-    TRY(dev_alloc(ctx, &ctx->d_rot, (ctx->mfma ? 1 : B) * ctx->R * ctx->S));
+    TRY(dev_alloc(ctx, &ctx->d_rot, ((ctx->mfma || ctx->mfma_sym) ? 1 : B) * ctx->R * ctx->S));
     TRY(dev_alloc(ctx, &ctx->d_key, B * ctx->N));
-    if (ctx->mfma) {
+    if (ctx->mfma_sym) {
+        TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->slices * 8 * ctx->KSs * 1024));
+        TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->slices * 8 * 32));
+        TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RTP * ctx->KSs * 1024));
+        TRY(dev_alloc(ctx, &ctx->d_nb, B * ctx->RTP * 32 * 8));
+    } else if (ctx->mfma) {
         TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->NT * ctx->KS * 1024));
         TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->NT * 32));
         TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RT * ctx->KS * 1024));
@@ -1218,8 +1317,44 @@ int run_dist_mfma(pink_hip_ctx *ctx, uint32_t B)
     return launch_check(ctx, "k_dist_mfma_u8");
 }
 
+int run_rotpack_sym(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
+{
+    Timed t(ctx, kClsRotate);
+    const size_t lds = (size_t)ctx->C * (ctx->I + 1) * (ctx->I + 1) * sizeof(float);
+    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(ctx->RTP * 4, B), dim3(256), lds, ctx->stream, dev_images, (v4i *)ctx->d_Pb,
+                       ctx->d_nb, ctx->d_cos, ctx->d_sin, ctx->d_upos, ctx->d_kmask, ctx->Ku, ctx->all_sym, ctx->C,
+                       ctx->I, ctx->nrr_eff, ctx->D, ctx->KSs, ctx->RTP);
+    return launch_check(ctx, "k_rotpack_sym_u8");
+}
+
+template <int KS>
+void launch_dist_sym(pink_hip_ctx *ctx, uint32_t B)
+{
+    const uint32_t groups = std::min(ctx->groups, B);
+    hipLaunchKernelGGL((k_dist_mfma_sym_u8<KS>), dim3(ctx->slices * groups), dim3(256), 0, ctx->stream,
+                       (const v4i *)ctx->d_Pa, ctx->d_na, (const v4i *)ctx->d_Pb, ctx->d_nb, ctx->d_key, ctx->N, B,
+                       ctx->cfg.num_rot, ctx->cfg.use_flip, ctx->nrr_eff, ctx->RTP, groups);
+}
+
+int run_dist_sym(pink_hip_ctx *ctx, uint32_t B)
+{
+    Timed t(ctx, kClsDist);
+    switch (ctx->KSs) {
+    case 8: launch_dist_sym<8>(ctx, B); break;
+    case 16: launch_dist_sym<16>(ctx, B); break;
+    case 24: launch_dist_sym<24>(ctx, B); break;
+    default: launch_dist_sym<32>(ctx, B); break;
+    }
+    return launch_check(ctx, "k_dist_mfma_sym_u8");
+}
+
 int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
+    if (ctx->mfma_sym) {
+        TRY(run_rotpack_sym(ctx, dev_images, B));
+        TRY(run_dist_sym(ctx, B));
+        return PINK_HIP_OK;
+    }
     if (ctx->mfma) {
         TRY(run_rotpack_mfma(ctx, dev_images, B));
         TRY(run_dist_mfma(ctx, B));

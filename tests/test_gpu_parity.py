@@ -90,10 +90,19 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
     s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, ed_type)
     rot = O.rotated_images(img, C_, I, D, nrot, flip)
     od, ossd, obest = O.distance_matrix(s, som, rot)
-    # a uint8 mapper runs on the matrix cores by default (N <= 128): check both kernels
-    choices = [capi.KERNEL_AUTO, capi.KERNEL_VALU] if ed_type == capi.UINT8 else [capi.KERNEL_AUTO]
+    # a uint8 mapper runs on the matrix cores where a kernel applies: check every kernel
+    choices = [capi.KERNEL_AUTO]
+    if ed_type == capi.UINT8:
+        choices += [capi.KERNEL_VALU, capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM]
+    ran = 0
     for choice in choices:
-        with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type, kernel_choice=choice) as ctx:
+        try:
+            ctx = capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type, kernel_choice=choice)
+        except capi.PinkError:
+            assert choice in (capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM)    # refused: shape outside that kernel
+            continue
+        ran += 1
+        with ctx:
             ctx.set_som(som)
             assert ctx.region_size == len(O.region(C_, D, ed, shape_))
             d, ssd, best = ctx.distance(img)
@@ -170,7 +179,8 @@ def test_reference_trainer_known_answers():
 
 
 MAP_CASES = [("cfg1", 24, None, capi.KERNEL_AUTO), ("cfg1", 9, None, capi.KERNEL_VALU),
-             ("cfg1", 3, None, capi.KERNEL_MFMA), ("cfg0", 5, capi.FLOAT, capi.KERNEL_AUTO),
+             ("cfg1", 13, None, capi.KERNEL_MFMA), ("cfg1", 40, None, capi.KERNEL_MFMA_SYM),
+             ("cfg0", 5, capi.FLOAT, capi.KERNEL_AUTO),
              ("cfg4", 300, None, capi.KERNEL_AUTO), ("cfg4", 50, None, capi.KERNEL_VALU),
              ("cfg2", 2, None, capi.KERNEL_AUTO)]
 
