@@ -57,7 +57,10 @@ def main():
     ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma"])
+    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma", "mfma_sym"])
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run one plain device-to-device copy of this many MiB (a kernel of known "
+                         "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (every figure is a "
@@ -73,7 +76,8 @@ def main():
     dev = torch.device("cuda:0")
     w = synthetic.WORKLOADS[args.workload]
     n_images = args.images or w.n_images
-    kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA}[args.kernel]
+    kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA,
+                     "mfma_sym": capi.KERNEL_MFMA_SYM}[args.kernel]
 
     t0 = time.time()
     imgs_host = synthetic.images(w, n_images)
@@ -95,6 +99,12 @@ def main():
     d_best = torch.empty((n_images, w.som_size), dtype=torch.int32, device=dev)
     d_bmu = torch.empty((n_images,), dtype=torch.int32, device=dev)
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        src = torch.empty(args.calibrate_copy << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)            # reads and writes exactly calibrate_copy MiB each
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         if w.mode == "map":

@@ -1177,6 +1177,7 @@ int init_ctx(pink_hip_ctx *ctx)
             for (uint32_t sym = 0; sym < 8; ++sym) if (sym_valid[sym]) valid_bits |= (unsigned char)(1u << sym);
             ctx->all_sym = 1;
             for (uint32_t k = 0; k < ctx->Ku; ++k) if ((kmask[k] & valid_bits) != valid_bits) ctx->all_sym = 0;
+            upos.resize(Kp, 0u);                       // padded: the kernel reads whole 16-entry pieces
             TRY(dev_alloc(ctx, &ctx->d_upos, upos.size()));
             TRY(dev_alloc(ctx, &ctx->d_aoff, aoff.size()));
             TRY(dev_alloc(ctx, &ctx->d_kmask, kmask.size()));
@@ -1321,9 +1322,10 @@ int run_rotpack_sym(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
     Timed t(ctx, kClsRotate);
     const size_t lds = (size_t)ctx->C * (ctx->I + 1) * (ctx->I + 1) * sizeof(float);
-    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(ctx->RTP * 4, B), dim3(256), lds, ctx->stream, dev_images, (v4i *)ctx->d_Pb,
+    const uint32_t blocks = ((B + 7) / 8) * 8 * ctx->RTP;          // 8 images per span of ids, see the kernel
+    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(blocks), dim3(256), lds, ctx->stream, dev_images, (v4i *)ctx->d_Pb,
                        ctx->d_nb, ctx->d_cos, ctx->d_sin, ctx->d_upos, ctx->d_kmask, ctx->Ku, ctx->all_sym, ctx->C,
-                       ctx->I, ctx->nrr_eff, ctx->D, ctx->KSs, ctx->RTP);
+                       ctx->I, ctx->nrr_eff, ctx->D, ctx->KSs, ctx->RTP, B);
     return launch_check(ctx, "k_rotpack_sym_u8");
 }
 
