@@ -32,13 +32,35 @@ FP32_PEAK_TFLOPS = 157.3       # MI355X vector fp32 (packed FMA), published
 DTYPE_NAME = {0: "f32", 1: "u16", 2: "u8"}
 
 
-def algorithmic_per_image(w, E):
-    """Algorithmic bytes / operations per image for each kernel class."""
+# Peaks measured on the MI355X box used for this work with small microbenchmarks (independent
+# MFMA / fma streams on all CUs): the clock settles near 2.0-2.2 GHz under load.  Reported next to
+# the published figures, never instead of them.
+MEASURED_INT8_MFMA_TOPS = 4130.0
+MEASURED_FMA_NOPACK_TFLOPS = 72.5
+
+# HBM bytes per image from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/cfg1_map_u8_hbm_traffic.txt),
+# scaled by the same counters' readings for a 256 MiB device-to-device copy (FETCH x2.0, WRITE x1.0).
+MEASURED_TRAFFIC_PER_IMAGE = {
+    ("cfg1", 3, "rotate"): 17.0e3 + 108.9e3,
+    ("cfg1", 3, "distance"): 108.1e3 + 0.8e3,
+}
+
+
+def algorithmic_per_image(w, E, path):
+    """Algorithmic bytes / operations per image for each kernel class.  `path` is the distance
+    kernel in use (capi.KERNEL_VALU / _MFMA / _MFMA_SYM): the matrix-core paths never write the
+    float variants, their rotation kernel emits the packed distance operand directly."""
     elem = {0: 4, 1: 2, 2: 1}[w.ed_type]
     S, R, N = w.neuron_size, w.R, w.som_size
+    nrr = max(w.num_rot // 4, 1)
+    kp = -(-E // 64) * 64
+    rot_bytes = R * S * 4 + w.image_size * 4              # all variants written once, image read once
+    if path == 2:      # uint8 MFMA, symmetries on the image side: ceil(nrr/4) tiles of 32 rows + norms
+        rot_bytes = w.image_size * 4 + -(-nrr // 4) * 32 * (kp + 4)
+    elif path == 3:    # uint8 MFMA, symmetries on the SOM side: ceil(nrr/32) tiles of 32 rows + 8 norms per row
+        rot_bytes = w.image_size * 4 + -(-nrr // 32) * 32 * (kp + 32)
     return {
-        # write all variants once, read the image once
-        "rotate": {"bytes": R * S * 4 + w.image_size * 4},
+        "rotate": {"bytes": rot_bytes},
         # region of every variant read as float32 and written in the distance type
         "pack": {"bytes": R * E * (4 + elem)},
         # every operand element read once; one subtract-square-accumulate = 2 operations
@@ -143,30 +165,59 @@ def main():
     ctx.set_profiling(False)
 
     value = n_images * args.steps / elapsed
-    alg = algorithmic_per_image(w, E)
+    path = ctx.distance_kernel
+    alg = algorithmic_per_image(w, E, path)
     total_ms = sum(ms for _, ms in times.values()) or 1e-9
     dominant = max(times, key=lambda k: times[k][1])
     launches, ms = times[dominant]
     avg_ms = ms / max(launches, 1)
     imgs_per_launch = prof_images / max(launches, 1)
+    per_s = imgs_per_launch / (avg_ms * 1e-3)
+    notes = None
     if dominant == "distance" and w.ed_type == capi.FLOAT:
-        # direct float32 form: sub + fma per pair element on the vector ALU, 2 ops counted per pair
+        # direct float32 form on the vector ALU: subtract + fma per pair element, counted as 2 ops
         bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
-        achieved = alg["distance"]["ops"] * imgs_per_launch / (avg_ms * 1e-3) / 1e12
+        achieved = alg["distance"]["ops"] * per_s / 1e12
+        notes = ("compute bound on the vector ALU, not on MFMA: bit-faithful sequential fma per (neuron, rotation); "
+                 "packed FP32 is disabled in this build, so the attainable rate is half the published "
+                 "157.3 TFLOP/s (measured %.1f TFLOP/s fma)" % MEASURED_FMA_NOPACK_TFLOPS)
+    elif dominant == "distance" and path == capi.KERNEL_MFMA_SYM:
+        bound, unit, peak = "mfma", "TOP/s", MFMA_INT8_PEAK_TOPS
+        achieved = alg["distance"]["ops"] * per_s / 1e12
+        notes = "int8 MFMA; measured MFMA peak on this box %.0f TOP/s" % MEASURED_INT8_MFMA_TOPS
     else:
         bound, unit, peak = "hbm", "GB/s", HBM_PEAK_GBS
-        achieved = alg[dominant]["bytes"] * imgs_per_launch / (avg_ms * 1e-3) / 1e9
+        achieved = alg[dominant]["bytes"] * per_s / 1e9
+        if dominant == "rotate" and path != capi.KERNEL_VALU:
+            notes = ("vector-ALU bound (exact bilinear arithmetic per operand byte), far from HBM: "
+                     "algorithmic bytes = image read + packed operand written")
+    traffic = MEASURED_TRAFFIC_PER_IMAGE.get((args.workload, path, dominant))
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-        "frac": round(achieved / peak, 5), "traffic": None,
+        "frac": round(achieved / peak, 5),
+        "traffic": round(traffic * imgs_per_launch) if traffic else None,
+        "algorithmic_bytes_per_launch": round(alg[dominant]["bytes"] * imgs_per_launch),
         "avg_launch_ms": round(avg_ms, 6), "launches": launches, "images_per_launch": imgs_per_launch,
         "measured": "timed region" if profile_in_timed else "separate pass of %d images" % prof_images,
         "share_of_kernel_time": round(ms / total_ms, 4),
         "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
+        "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries"}[path],
     }
-    if "ops" in alg[dominant] and w.ed_type != capi.FLOAT:
-        roofline["mfma_int8_frac"] = round(
-            alg[dominant]["ops"] * imgs_per_launch / (avg_ms * 1e-3) / 1e12 / MFMA_INT8_PEAK_TOPS, 5)
+    if notes:
+        roofline["note"] = notes
+    # the distance kernel's own fractions, whichever kernel dominates
+    d_launches, d_ms = times["distance"]
+    if d_launches:
+        d_per_s = prof_images / (d_ms * 1e-3)
+        dist = {"ops_per_s": alg["distance"]["ops"] * d_per_s, "share_of_kernel_time": round(d_ms / total_ms, 4)}
+        if w.ed_type == capi.FLOAT:
+            dist["frac_of_fp32_157.3TF"] = round(dist["ops_per_s"] / 1e12 / FP32_PEAK_TFLOPS, 5)
+            dist["frac_of_measured_nopack_fma"] = round(dist["ops_per_s"] / 1e12 / MEASURED_FMA_NOPACK_TFLOPS, 5)
+        else:
+            dist["frac_of_int8_mfma_5POPs"] = round(dist["ops_per_s"] / 1e12 / MFMA_INT8_PEAK_TOPS, 5)
+            dist["hbm_frac_survey_bytes"] = round(alg["distance"]["bytes"] * d_per_s / 1e9 / HBM_PEAK_GBS, 5)
+        dist["ops_per_s"] = round(dist["ops_per_s"] / 1e12, 3)
+        roofline["distance_kernel"] = dist
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -141,6 +141,8 @@ int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_di
 
 /* Number of elements in the distance region (incl. channels) as the context counts it. */
 uint32_t pink_hip_region_size(const pink_hip_ctx *ctx);
+/* The distance kernel the context runs: PINK_HIP_KERNEL_VALU, _MFMA or _MFMA_SYM. */
+uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx);
 
 /* Per-kernel timing with HIP events on the context's stream.  While enabled every
  * launch of the rotation, distance and update kernels is bracketed by two events;

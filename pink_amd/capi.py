@@ -26,7 +26,7 @@ EXPORTS = (
     "pink_hip_abi_version", "pink_hip_create", "pink_hip_destroy", "pink_hip_last_error",
     "pink_hip_set_som", "pink_hip_get_som", "pink_hip_train", "pink_hip_train_device",
     "pink_hip_map", "pink_hip_map_device", "pink_hip_synchronize", "pink_hip_rotate",
-    "pink_hip_distance", "pink_hip_region_size", "pink_hip_set_profiling",
+    "pink_hip_distance", "pink_hip_region_size", "pink_hip_distance_kernel", "pink_hip_set_profiling",
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
     "pink_hip_make_update_factors",
 )
@@ -76,6 +76,8 @@ def lib():
         L.pink_hip_distance.argtypes = [vp, f32p, f32p, C.POINTER(C.c_int64), u32p]
         L.pink_hip_region_size.argtypes = [vp]
         L.pink_hip_region_size.restype = u32
+        L.pink_hip_distance_kernel.argtypes = [vp]
+        L.pink_hip_distance_kernel.restype = u32
         L.pink_hip_set_profiling.argtypes = [vp, C.c_int]
         L.pink_hip_kernel_times.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_double)]
         L.pink_hip_device_info.argtypes = [C.c_char_p, C.c_size_t]
@@ -170,6 +172,11 @@ class Context:
     @property
     def region_size(self):
         return int(self._L.pink_hip_region_size(self._h))
+
+    @property
+    def distance_kernel(self):
+        """KERNEL_VALU, KERNEL_MFMA or KERNEL_MFMA_SYM: the distance kernel this context runs."""
+        return int(self._L.pink_hip_distance_kernel(self._h))
 
     def set_som(self, som):
         som = np.ascontiguousarray(som, np.float32)

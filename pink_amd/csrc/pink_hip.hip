@@ -1615,6 +1615,12 @@ int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_di
 
 uint32_t pink_hip_region_size(const pink_hip_ctx *ctx) { return ctx ? ctx->E : 0; }
 
+uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx)
+{
+    if (!ctx) return 0;
+    return ctx->mfma_sym ? PINK_HIP_KERNEL_MFMA_SYM : ctx->mfma ? PINK_HIP_KERNEL_MFMA : PINK_HIP_KERNEL_VALU;
+}
+
 int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)
 {
     if (!ctx) return PINK_HIP_EINVAL;
