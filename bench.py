@@ -79,7 +79,7 @@ def main():
     ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma", "mfma_sym"])
+    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma", "mfma_sym", "mfma_gemm"])
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run one plain device-to-device copy of this many MiB (a kernel of known "
                          "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -99,7 +99,7 @@ def main():
     w = synthetic.WORKLOADS[args.workload]
     n_images = args.images or w.n_images
     kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA,
-                     "mfma_sym": capi.KERNEL_MFMA_SYM}[args.kernel]
+                     "mfma_sym": capi.KERNEL_MFMA_SYM, "mfma_gemm": capi.KERNEL_MFMA_GEMM}[args.kernel]
 
     t0 = time.time()
     imgs_host = synthetic.images(w, n_images)
@@ -201,7 +201,8 @@ def main():
         "measured": "timed region" if profile_in_timed else "separate pass of %d images" % prof_images,
         "share_of_kernel_time": round(ms / total_ms, 4),
         "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
-        "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries"}[path],
+        "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries",
+                          4: "int8 MFMA GEMM, split k"}[path],
     }
     if notes:
         roofline["note"] = notes

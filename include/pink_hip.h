@@ -63,7 +63,8 @@ typedef enum {
     PINK_HIP_KERNEL_AUTO = 0,      /* float32: sequential-fma vector-ALU kernel; uint8 mapper: int8 MFMA where it applies */
     PINK_HIP_KERNEL_VALU = 1,      /* integer modes on the vector ALU in exact int32/int64                */
     PINK_HIP_KERNEL_MFMA = 2,      /* uint8 mapper, int8 MFMA, symmetries applied to the image variants   */
-    PINK_HIP_KERNEL_MFMA_SYM = 3   /* uint8 mapper, int8 MFMA, symmetries applied to the SOM once         */
+    PINK_HIP_KERNEL_MFMA_SYM = 3,  /* uint8 mapper, int8 MFMA, symmetries applied to the SOM once         */
+    PINK_HIP_KERNEL_MFMA_GEMM = 4  /* integer modes, trainer or mapper: split-k int8 MFMA GEMM (uint16 as 4 byte-plane products) */
 } pink_hip_kernel_choice;
 
 /*
@@ -141,7 +142,7 @@ int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_di
 
 /* Number of elements in the distance region (incl. channels) as the context counts it. */
 uint32_t pink_hip_region_size(const pink_hip_ctx *ctx);
-/* The distance kernel the context runs: PINK_HIP_KERNEL_VALU, _MFMA or _MFMA_SYM. */
+/* The distance kernel the context runs: PINK_HIP_KERNEL_VALU, _MFMA, _MFMA_SYM or _MFMA_GEMM. */
 uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx);
 
 /* Per-kernel timing with HIP events on the context's stream.  While enabled every

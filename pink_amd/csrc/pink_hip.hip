@@ -653,6 +653,7 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
 }
 
 #include "mfma_u8_sym.inc"
+#include "mfma_int_gemm.inc"
 
 // ---------------------------------------------------------------------------------
 // BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
@@ -784,6 +785,13 @@ struct pink_hip_ctx {
     uint32_t *d_upos = nullptr, *d_aoff = nullptr;
     unsigned char *d_kmask = nullptr;
 
+    // integer distances as an int8 MFMA GEMM with split k (training, SOMs of any size)
+    bool gemm = false;
+    uint32_t gKS = 0, Np = 0, Rp = 0, gsplits = 1, gks_per = 0;
+    v4i *d_gPa = nullptr, *d_gPb = nullptr;
+    long long *d_gna = nullptr, *d_gnb = nullptr;
+    int *d_dot = nullptr;
+
     uint32_t force_tn = 0;     // tuning aid: PINK_HIP_DIST_TN=1|2|4|8 overrides the neurons-per-wave choice
 
     bool profiling = false;
@@ -909,6 +917,15 @@ bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT
 int run_pack_som(pink_hip_ctx *ctx)
 {
     Timed t(ctx, kClsPack);
+    if (ctx->gemm) {
+        if (ctx->cfg.ed_type == PINK_HIP_UINT16)
+            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+                               ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+        else
+            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+                               ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+        return launch_check(ctx, "k_pack_planes");
+    }
     if (ctx->mfma_sym) {
         hipLaunchKernelGGL(k_pack_som_sym_u8, dim3(ctx->slices * 8 * 32), dim3(256), 0, ctx->stream, ctx->d_som,
                            ctx->d_aoff, ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->KSs);
@@ -944,6 +961,15 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 {
     Timed t(ctx, kClsPack);
+    if (ctx->gemm) {
+        if (ctx->cfg.ed_type == PINK_HIP_UINT16)
+            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region,
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
+        else
+            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region,
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
+        return launch_check(ctx, "k_pack_planes");
+    }
     if (!is_int(ctx)) {
         hipLaunchKernelGGL(k_pack_rot_rows, dim3((ctx->Epad + 255) / 256, ctx->Rpad, B), dim3(256), 0, ctx->stream,
                            ctx->d_rot, ctx->d_region, (float *)ctx->d_rotT, ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad);
@@ -1006,9 +1032,30 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 #undef LAUNCH_TN
 }
 
+template <bool U16>
+void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot)
+{
+    const uint32_t planes = U16 ? 2 : 1;
+    const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
+    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(ctx->Rp / 64, ctx->Np / 64, ctx->gsplits), dim3(64), 0, ctx->stream,
+                       ctx->d_gPa, pb, ctx->d_dot, ctx->N, ctx->Np, ctx->R, ctx->Rp, ctx->gKS, ctx->gks_per);
+    hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32), dim3(256), 0, ctx->stream, ctx->d_dot,
+                       ctx->d_gna, ctx->d_gnb + (size_t)slot * ctx->Rp, ctx->d_key + (size_t)slot * ctx->N, ctx->N,
+                       ctx->Np, ctx->R, ctx->Rp);
+}
+
 int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     Timed t(ctx, kClsDist);
+    if (ctx->gemm) {
+        for (uint32_t b = 0; b < B; ++b) {
+            if (ctx->cfg.ed_type == PINK_HIP_UINT16) launch_dist_gemm<true>(ctx, slot + b);
+            else launch_dist_gemm<false>(ctx, slot + b);
+        }
+        return launch_check(ctx, "k_dist_gemm_int");
+    }
+    // the vector-ALU kernels below read d_somP / d_rotT: never reached without them
+    if (!ctx->d_somP || !ctx->d_rotT) return fail(ctx, PINK_HIP_ESTATE, "distance operands were not allocated");
     switch (ctx->cfg.ed_type) {
     case PINK_HIP_FLOAT: launch_dist_f32(ctx, slot, B); break;
     case PINK_HIP_UINT8: launch_dist<1>(ctx, slot, B); break;
@@ -1024,7 +1071,7 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
     hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
-                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP, ctx->d_inv, ctx->Epad,
+                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP, ctx->gemm ? nullptr : ctx->d_inv, ctx->Epad,
                        is_int(ctx) ? (float)ctx->factor : 0.0f);
     return launch_check(ctx, "k_update");
 }
@@ -1048,7 +1095,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -1224,9 +1271,32 @@ int init_ctx(pink_hip_ctx *ctx)
         HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_dist));
     }
 
+    // Integer distances as a split-k int8 GEMM: what is left of the integer modes when the SOM is
+    // large enough to fill 64 x 64 tiles (smaller problems are latency bound either way).
+    {
+        const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->E <= 131071;
+        if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM && !applies)
+            return fail(ctx, PINK_HIP_EINVAL, "the MFMA GEMM distance kernel needs an integer distance type");
+        ctx->gemm = applies && (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM ||
+                                (c.kernel_choice == PINK_HIP_KERNEL_AUTO && ctx->N >= 64 && ctx->R >= 64));
+        if (ctx->gemm) {
+            ctx->gKS = ctx->Epad / 32;
+            ctx->Np = round_up(ctx->N, 64);
+            ctx->Rp = round_up(ctx->R, 64);
+            const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
+            uint32_t splits = std::max(1u, (2u * (uint32_t)ctx->num_cu + tiles - 1) / tiles);
+            splits = std::min(splits, std::max(1u, ctx->gKS / 4));
+            ctx->gks_per = (ctx->gKS + splits - 1) / splits;
+            ctx->gsplits = (ctx->gKS + ctx->gks_per - 1) / ctx->gks_per;
+        }
+    }
+
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
     size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
     if (ctx->mfma) per_image = (size_t)ctx->RT * ctx->KS * 1024 + (size_t)ctx->RT * 128 + (size_t)ctx->N * 24;
+    if (ctx->gemm)
+        per_image = (size_t)ctx->R * ctx->S * 4 + (size_t)(c.ed_type == PINK_HIP_UINT16 ? 2 : 1) * (ctx->Rp / 32) * ctx->gKS * 1024 +
+                    (size_t)ctx->Rp * 8 + (size_t)ctx->N * 24;
     if (ctx->mfma_sym) per_image = (size_t)ctx->RTP * ctx->KSs * 1024 + (size_t)ctx->RTP * 32 * 8 * 4 + (size_t)ctx->N * 24;
     if (ctx->trainer) {
         // images whose variants are prepared ahead of the sequential distance/update chain
@@ -1254,6 +1324,19 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->slices * 8 * 32));
         TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RTP * ctx->KSs * 1024));
         TRY(dev_alloc(ctx, &ctx->d_nb, B * ctx->RTP * 32 * 8));
+    } else if (ctx->gemm) {
+        const size_t planes = c.ed_type == PINK_HIP_UINT16 ? 2 : 1;
+        const size_t a_vec = planes * (ctx->Np / 32) * ctx->gKS * 64, b_vec = planes * (ctx->Rp / 32) * ctx->gKS * 64;
+        const size_t dot_n = (planes == 2 ? 3 : 1) * (size_t)ctx->Rp * ctx->Np;
+        TRY(dev_alloc(ctx, &ctx->d_gPa, a_vec));
+        TRY(dev_alloc(ctx, &ctx->d_gPb, B * b_vec));
+        TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)ctx->Np));
+        TRY(dev_alloc(ctx, &ctx->d_gnb, B * ctx->Rp));
+        TRY(dev_alloc(ctx, &ctx->d_dot, dot_n));
+        // rows beyond N / R and elements beyond the region are never written: they must read as zero
+        HIP_TRY(ctx, hipMemset(ctx->d_gPa, 0, a_vec * sizeof(v4i)));
+        HIP_TRY(ctx, hipMemset(ctx->d_gPb, 0, B * b_vec * sizeof(v4i)));
+        HIP_TRY(ctx, hipMemset(ctx->d_dot, 0, dot_n * sizeof(int)));
     } else if (ctx->mfma) {
         TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->NT * ctx->KS * 1024));
         TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->NT * 32));
@@ -1482,7 +1565,7 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
         for (uint32_t b = 0; b < B; ++b) {
             TRY(run_dist(ctx, b, 1));
             TRY(run_update(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
-            if (!ctx->d_inv) TRY(run_pack_som(ctx));
+            if (!ctx->d_inv || ctx->gemm) TRY(run_pack_som(ctx));
         }
     }
     return PINK_HIP_OK;
@@ -1618,7 +1701,8 @@ uint32_t pink_hip_region_size(const pink_hip_ctx *ctx) { return ctx ? ctx->E : 0
 uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx)
 {
     if (!ctx) return 0;
-    return ctx->mfma_sym ? PINK_HIP_KERNEL_MFMA_SYM : ctx->mfma ? PINK_HIP_KERNEL_MFMA : PINK_HIP_KERNEL_VALU;
+    return ctx->mfma_sym ? PINK_HIP_KERNEL_MFMA_SYM : ctx->mfma ? PINK_HIP_KERNEL_MFMA
+         : ctx->gemm ? PINK_HIP_KERNEL_MFMA_GEMM : PINK_HIP_KERNEL_VALU;
 }
 
 int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)

@@ -93,7 +93,9 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
     # a uint8 mapper runs on the matrix cores where a kernel applies: check every kernel
     choices = [capi.KERNEL_AUTO]
     if ed_type == capi.UINT8:
-        choices += [capi.KERNEL_VALU, capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM]
+        choices += [capi.KERNEL_VALU, capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA_GEMM]
+    if ed_type == capi.UINT16:
+        choices += [capi.KERNEL_VALU, capi.KERNEL_MFMA_GEMM]
     ran = 0
     for choice in choices:
         try:
@@ -116,21 +118,24 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
 
 
 TRAIN_CASES = [
-    # workload, images, ed_type override
-    ("cfg0", 6, None), ("cfg4", 40, None), ("cfg0", 4, capi.UINT8), ("cfg2", 2, None), ("cfg3", 1, None),
+    # workload, images, ed_type override, distance kernel
+    ("cfg0", 6, None, capi.KERNEL_AUTO), ("cfg4", 40, None, capi.KERNEL_AUTO), ("cfg4", 10, None, capi.KERNEL_MFMA_GEMM),
+    ("cfg0", 4, capi.UINT8, capi.KERNEL_AUTO), ("cfg0", 3, capi.UINT8, capi.KERNEL_VALU),
+    ("cfg0", 3, capi.UINT16, capi.KERNEL_AUTO), ("cfg2", 3, None, capi.KERNEL_AUTO), ("cfg2", 1, None, capi.KERNEL_VALU),
+    ("cfg3", 1, None, capi.KERNEL_AUTO),
 ]
 
 
-@pytest.mark.parametrize("name,n,ed_type", TRAIN_CASES)
-def test_train_parity(name, n, ed_type):
+@pytest.mark.parametrize("name,n,ed_type,choice", TRAIN_CASES)
+def test_train_parity(name, n, ed_type, choice):
     w = synthetic.WORKLOADS[name]
     ed_type = w.ed_type if ed_type is None else ed_type
-    say("train", name, n, ed_type)
+    say("train", name, n, ed_type, choice)
     imgs = synthetic.images(w, n)
     som0 = synthetic.initial_som(w)
     F = synthetic.update_factors(w)
     with capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
-                      w.ed_shape, ed_type, F) as ctx:
+                      w.ed_shape, ed_type, F, kernel_choice=choice) as ctx:
         ctx.set_som(som0)
         bmu = ctx.train(imgs)
         got = ctx.get_som()
