@@ -787,7 +787,7 @@ struct pink_hip_ctx {
 
     // integer distances as an int8 MFMA GEMM with split k (training, SOMs of any size)
     bool gemm = false;
-    uint32_t gKS = 0, Np = 0, Rp = 0, gsplits = 1, gks_per = 0;
+    uint32_t gKS = 0, Np = 0, Rp = 0, gslices = 1, gks_per = 0;   // k-slices (blocks per tile), k-steps per wave
     v4i *d_gPa = nullptr, *d_gPb = nullptr;
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
@@ -919,10 +919,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     Timed t(ctx, kClsPack);
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
-            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(1024), 2 * ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
                                ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
         else
-            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
+            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(1024), ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
                                ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
         return launch_check(ctx, "k_pack_planes");
     }
@@ -963,10 +963,10 @@ int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
     Timed t(ctx, kClsPack);
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
-            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region,
+            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(256), 2 * ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
                                ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
         else
-            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region,
+            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(256), ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
                                ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
         return launch_check(ctx, "k_pack_planes");
     }
@@ -1037,11 +1037,13 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot)
 {
     const uint32_t planes = U16 ? 2 : 1;
     const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
-    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(ctx->Rp / 64, ctx->Np / 64, ctx->gsplits), dim3(64), 0, ctx->stream,
-                       ctx->d_gPa, pb, ctx->d_dot, ctx->N, ctx->Np, ctx->R, ctx->Rp, ctx->gKS, ctx->gks_per);
-    hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32), dim3(256), 0, ctx->stream, ctx->d_dot,
-                       ctx->d_gna, ctx->d_gnb + (size_t)slot * ctx->Rp, ctx->d_key + (size_t)slot * ctx->N, ctx->N,
-                       ctx->Np, ctx->R, ctx->Rp);
+    const uint32_t tiles_per_xcd = ((ctx->Rp / 64) * (ctx->Np / 64) + 7) / 8;
+    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * ctx->gslices), dim3(256), 0, ctx->stream, ctx->d_gPa, pb,
+                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ctx->gks_per, ctx->gslices, tiles_per_xcd);
+    const uint32_t rows_per_chunk = 32;
+    hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
+                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, ctx->d_gna, ctx->d_gnb + (size_t)slot * ctx->Rp,
+                       ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Np, ctx->R, ctx->Rp, ctx->gslices, rows_per_chunk);
 }
 
 int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
@@ -1274,7 +1276,7 @@ int init_ctx(pink_hip_ctx *ctx)
     // Integer distances as a split-k int8 GEMM: what is left of the integer modes when the SOM is
     // large enough to fill 64 x 64 tiles (smaller problems are latency bound either way).
     {
-        const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->E <= 131071;
+        const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->Epad <= 32768;   // planes of a row fit LDS
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM && !applies)
             return fail(ctx, PINK_HIP_EINVAL, "the MFMA GEMM distance kernel needs an integer distance type");
         ctx->gemm = applies && (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM ||
@@ -1284,10 +1286,12 @@ int init_ctx(pink_hip_ctx *ctx)
             ctx->Np = round_up(ctx->N, 64);
             ctx->Rp = round_up(ctx->R, 64);
             const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
-            uint32_t splits = std::max(1u, (2u * (uint32_t)ctx->num_cu + tiles - 1) / tiles);
-            splits = std::min(splits, std::max(1u, ctx->gKS / 4));
-            ctx->gks_per = (ctx->gKS + splits - 1) / splits;
-            ctx->gsplits = (ctx->gKS + ctx->gks_per - 1) / ctx->gks_per;
+            // k is cut so that every CU gets about two waves; a block of four waves takes one slice
+            uint32_t cuts = std::max(1u, (2u * (uint32_t)ctx->num_cu + tiles - 1) / tiles);
+            cuts = std::min(cuts, std::max(1u, ctx->gKS / 4));
+            const uint32_t slices = (cuts + 3) / 4;
+            ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
+            ctx->gslices = (ctx->gKS + 4 * ctx->gks_per - 1) / (4 * ctx->gks_per);
         }
     }
 
@@ -1327,7 +1331,7 @@ int init_ctx(pink_hip_ctx *ctx)
     } else if (ctx->gemm) {
         const size_t planes = c.ed_type == PINK_HIP_UINT16 ? 2 : 1;
         const size_t a_vec = planes * (ctx->Np / 32) * ctx->gKS * 64, b_vec = planes * (ctx->Rp / 32) * ctx->gKS * 64;
-        const size_t dot_n = (planes == 2 ? 3 : 1) * (size_t)ctx->Rp * ctx->Np;
+        const size_t dot_n = ctx->gslices * planes * (size_t)ctx->Rp * ctx->Np;   // int32 (uint8) or int64 (uint16) per element
         TRY(dev_alloc(ctx, &ctx->d_gPa, a_vec));
         TRY(dev_alloc(ctx, &ctx->d_gPb, B * b_vec));
         TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)ctx->Np));
