@@ -1273,14 +1273,15 @@ int init_ctx(pink_hip_ctx *ctx)
         HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_dist));
     }
 
-    // Integer distances as a split-k int8 GEMM: what is left of the integer modes when the SOM is
-    // large enough to fill 64 x 64 tiles (smaller problems are latency bound either way).
+    // Integer distances as a split-k int8 GEMM: all that is left of the integer modes.  Small
+    // problems pad their rows to one 64 x 64 tile; they are latency bound either way and the four
+    // waves of a block still cut k four ways.
     {
         const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->Epad <= 32768;   // planes of a row fit LDS
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM && !applies)
             return fail(ctx, PINK_HIP_EINVAL, "the MFMA GEMM distance kernel needs an integer distance type");
         ctx->gemm = applies && (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM ||
-                                (c.kernel_choice == PINK_HIP_KERNEL_AUTO && ctx->N >= 64 && ctx->R >= 64));
+                                c.kernel_choice == PINK_HIP_KERNEL_AUTO);
         if (ctx->gemm) {
             ctx->gKS = ctx->Epad / 32;
             ctx->Np = round_up(ctx->N, 64);

@@ -119,7 +119,7 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
 
 TRAIN_CASES = [
     # workload, images, ed_type override, distance kernel
-    ("cfg0", 6, None, capi.KERNEL_AUTO), ("cfg4", 40, None, capi.KERNEL_AUTO), ("cfg4", 10, None, capi.KERNEL_MFMA_GEMM),
+    ("cfg0", 6, None, capi.KERNEL_AUTO), ("cfg4", 40, None, capi.KERNEL_AUTO), ("cfg4", 10, None, capi.KERNEL_VALU),
     ("cfg0", 4, capi.UINT8, capi.KERNEL_AUTO), ("cfg0", 3, capi.UINT8, capi.KERNEL_VALU),
     ("cfg0", 3, capi.UINT16, capi.KERNEL_AUTO), ("cfg2", 3, None, capi.KERNEL_AUTO), ("cfg2", 1, None, capi.KERNEL_VALU),
     ("cfg3", 1, None, capi.KERNEL_AUTO),
