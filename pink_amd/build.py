@@ -14,6 +14,12 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(HERE, "csrc", "pink_hip.hip"), os.path.join(HERE, "csrc", "update_factors.cpp")]
+# Compiled on its own with the MFMA accumulators in the architectural vector registers: its
+# distance kernel fills all 256 accumulation registers with resident SOM fragments (which the MFMA
+# reads as operands) and post-processes the accumulators on the vector ALU, which cannot read
+# accumulation registers.  The other MFMA kernels want the default (accumulators there).
+SYM_SOURCE = os.path.join(HERE, "csrc", "mfma_u8_sym.hip")
+SYM_FLAGS = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
 OUT = os.path.join(HERE, "lib", "libpink_hip.so")
 
 HIPCC_FLAGS = [
@@ -28,10 +34,18 @@ HIPCC_FLAGS = [
 def build(verbose=False, extra=()):
     os.makedirs(os.path.dirname(OUT), exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + list(extra) + SOURCES + ["-o", OUT]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    obj_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objects, cmds = [], []
+    for src in SOURCES + [SYM_SOURCE]:
+        obj = os.path.join(HERE, "lib", os.path.splitext(os.path.basename(src))[0] + ".o")
+        flags = obj_flags + (SYM_FLAGS if src == SYM_SOURCE else [])
+        cmds.append([hipcc] + flags + list(extra) + ["-c", src, "-o", obj])
+        objects.append(obj)
+    cmds.append([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", OUT])
+    for cmd in cmds:
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
     return OUT
 
 

@@ -1,0 +1,499 @@
+// mfma_u8_sym.hip -- uint8 mapping with the 8 symmetries moved to the SOM side.
+// A translation unit of its own: it is compiled with MFMA accumulators in the architectural
+// vector registers, so that the accumulation registers can hold the resident SOM fragments
+// (see the build script); pink_hip.hip reaches it through the launchers in mfma_u8_sym.h.
+//
+// A mapper's SOM never changes, so the quarter turns and the flip are applied to the
+// neurons once instead of to every image: with perm_s the map from variant coordinates to
+// base-rotation coordinates of symmetry s,
+//   ssd(n, variant (s, i)) = sum_{e in region} (q_n[off_e] - q_i[perm_s(off_e)])^2
+//                          = sum_{p in P_s} (A_{n,s}[p] - q_i[p])^2,   P_s = perm_s(region),
+// where q_i is the quantised base rotation i (0 <= angle < 90 degrees) and A_{n,s}[p] is the
+// neuron element that symmetry s pairs with base position p.  Over the union U of the P_s,
+// with A_{n,s} = 0 outside P_s (values shifted by -128),
+//   ssd = |A_{n,s}|^2 + sum_{p in P_s} q'_i[p]^2 - 2 A_{n,s} . q'_i          (exact in int32).
+// The image side shrinks to num_rot/4 rows per image (8x fewer bytes to produce and to
+// stream); the SOM side grows to 8 rows per neuron, prepared once.
+//
+// Operands are fragment-major as in the other matrix-core path: rows in tiles of 32, k in
+// steps of 32, a (tile, k-step) fragment = 64 lanes x 16 bytes, lane l = row l % 32,
+// k-half l / 32.  SOM-side rows are m = n * 8 + s, so the 8 symmetries of a neuron sit in 8
+// adjacent lanes of the MFMA's column operand.
+
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+
+#include "mfma_u8_sym.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// q = T(x * factor) saturated to [0, factor] (CudaLib/copy_and_transform_kernel.h:27-28)
+__device__ __forceinline__ int32_t quantise(float x, float factor)
+{
+    const float v = __fmul_rn(x, factor);
+    if (!(v > 0.0f)) return 0;
+    if (v >= factor) return (int32_t)factor;
+    return (int32_t)v;
+}
+
+// SOM operand.  One block per row m = n * 8 + s (rows beyond 8 N are zero).
+// aoff[s][k] = neuron element paired with union position k under symmetry s, or ~0.
+__global__ __launch_bounds__(256) void k_pack_som_sym_u8(const float *__restrict__ som, const uint32_t *__restrict__ aoff,
+                                                         signed char *__restrict__ Pa, int *__restrict__ na, uint32_t N,
+                                                         uint32_t S, uint32_t KS)
+{
+    __shared__ int s_sum[256];
+    const uint32_t m = blockIdx.x, n = m >> 3, sym = m & 7;
+    const uint32_t Kp = KS * 32;
+    int sq = 0;
+    for (uint32_t k = threadIdx.x; k < Kp; k += 256) {
+        int v = 0;
+        if (n < N) {
+            const uint32_t o = aoff[(size_t)sym * Kp + k];
+            if (o != 0xffffffffu) v = quantise(som[(size_t)n * S + o], 255.0f) - 128;
+        }
+        sq += v * v;
+        const uint32_t lane = (m & 31) + 32 * ((k & 31) >> 4);
+        Pa[((((size_t)(m >> 5) * KS + (k >> 5)) * 64 + lane) << 4) + (k & 15)] = (signed char)v;
+    }
+    s_sum[threadIdx.x] = sq;
+    __syncthreads();
+    for (uint32_t s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) s_sum[threadIdx.x] += s_sum[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) na[m] = s_sum[0];
+}
+
+// Image operand: base rotations only.  A block handles one row tile (32 base rotations) of one
+// image.  The image is staged in LDS with one extra zero column per row and one extra zero row per
+// channel, so the two neighbours that the bilinear rule reads with weight 0 at the last
+// row / column (ImageProcessingLib/rotate.h:50,62-63) need no index clamp.  A thread evaluates
+// 16 consecutive union positions of one rotation (bilinear in the CPU's operation order,
+// quantised, shifted), stores them as one 16-byte piece of a fragment, and adds their squares
+// to the 8 per-symmetry norms of that rotation according to kmask (bit s of kmask[k] set when
+// union position k belongs to P_s).
+//   upos[k] = (channel << 24 | x << 12 | y) of union element k, k < Ku (0 beyond, up to KS * 32).
+// Bilinear value of base rotation i > 0 at the neuron pixel whose centred coordinates are
+// (px, py) = (x - (D-1)/2, y - (D-1)/2), from the padded LDS image.  Branch-free: the taps are
+// read at the clamped position and the result is replaced by 0 when the source position lies
+// outside the image (ImageProcessingLib/rotate.h:40-44), so a wave never diverges here.
+__device__ __forceinline__ float bilinear_lds(const float *__restrict__ s_img, uint32_t W, float src_c, float lim,
+                                              float cs, float sn, float px, float py)
+{
+    const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+    const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+    const bool outside = sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim;
+    const float sxc = __builtin_amdgcn_fmed3f(sxf, 0.0f, lim), syc = __builtin_amdgcn_fmed3f(syf, 0.0f, lim);
+    const uint32_t ix = (uint32_t)sxc, iy = (uint32_t)syc;
+    const float rx = __fsub_rn(sxc, (float)ix), ry = __fsub_rn(syc, (float)iy);
+    const float cx = __fsub_rn(1.0f, rx), cy = __fsub_rn(1.0f, ry);
+    const float *t = s_img + ix * W + iy;
+    const float a = __fmul_rn(__fmul_rn(cx, cy), t[0]);
+    const float b = __fmul_rn(__fmul_rn(cx, ry), t[1]);
+    const float c = __fmul_rn(__fmul_rn(rx, cy), t[W]);
+    const float d = __fmul_rn(__fmul_rn(rx, ry), t[W + 1]);
+    const float v = __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
+    return outside ? 0.0f : v;
+}
+
+// Centre crop / centre pad (base rotation 0), ImageProcessingLib/resize.h:15-40.
+__device__ __forceinline__ float resize_lds(const float *__restrict__ s_img, uint32_t W, uint32_t I, uint32_t D,
+                                            uint32_t x, uint32_t y)
+{
+    if (I >= D) {
+        const uint32_t m = (I - D) / 2;
+        return s_img[(x + m) * W + (y + m)];
+    }
+    const uint32_t m = (D - I) / 2;
+    const uint32_t sx = x - m, sy = y - m;
+    return (sx < I && sy < I) ? s_img[sx * W + sy] : 0.0f;
+}
+
+// q = uint8(x * 255) saturated (NaN -> 0): multiply, clamp (v_med3_f32), convert.
+__device__ __forceinline__ uint32_t quantise_u8(float x)
+{
+    return (uint32_t)__builtin_amdgcn_fmed3f(__fmul_rn(x, 255.0f), 0.0f, 255.0f);
+}
+
+__global__ __launch_bounds__(256) void k_rotpack_sym_u8(const float *__restrict__ images, v4i *__restrict__ Pb,
+                                                        const float *__restrict__ cos_t,
+                                                        const float *__restrict__ sin_t,
+                                                        const uint32_t *__restrict__ upos,
+                                                        const unsigned char *__restrict__ kmask, uint32_t Ku,
+                                                        uint32_t all_sym, uint32_t C, uint32_t I, uint32_t nrr_eff,
+                                                        uint32_t D, uint32_t KS, uint32_t RTP, uint32_t B)
+{
+    extern __shared__ float s_img[];                      // C x (I + 1) x (I + 1), zero padded
+    const uint32_t UNIT_V = KS * 64 + 64;                 // 16-byte vectors per unit: fragments, then norm entries
+    __shared__ int s_nb[32][8];
+    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The
+    // id is decoded so that all blocks of one image share id % 8, i.e. one XCD: the image then
+    // leaves HBM once instead of once per XCD.
+    const uint32_t lin = blockIdx.x;
+    const uint32_t span = 8 * RTP;                        // ids covering 8 images
+    const uint32_t rt = (lin % span) / 8;
+    const uint32_t b = (lin / span) * 8 + (lin % 8);
+    if (b >= B) return;
+    const uint32_t W = I + 1, CH = W * W, II = I * I;
+    const float *img = images + (size_t)b * C * II;
+    s_nb[threadIdx.x >> 3][threadIdx.x & 7] = 0;
+    for (uint32_t c = 0; c < C; ++c) {
+        // coalesced copy of the I x I channel into the padded tile; (r, q) advance without divisions
+        uint32_t r = threadIdx.x / I, q = threadIdx.x % I;
+        for (uint32_t t = threadIdx.x; t < II; t += 256) {
+            s_img[c * CH + r * W + q] = img[(size_t)c * II + t];
+            q += 256;
+            while (q >= I) { q -= I; ++r; }
+        }
+        for (uint32_t t = threadIdx.x; t <= I; t += 256) {
+            s_img[c * CH + t * W + I] = 0.0f;             // extra column
+            s_img[c * CH + I * W + t] = 0.0f;             // extra row
+        }
+    }
+    __syncthreads();
+
+    const float src_c = __fmul_rn((float)(I - 1), 0.5f), dst_c = __fmul_rn((float)(D - 1), 0.5f);
+    const float lim = (float)(I - 1);
+    const uint32_t pieces = KS * 2;                       // 16-element pieces per row
+    for (uint32_t t = threadIdx.x; t < 32 * pieces; t += blockDim.x) {
+        const uint32_t g = t / pieces, piece = t % pieces;
+        const uint32_t i = rt * 32 + g;                   // base rotation
+        const uint32_t k0 = piece * 16;
+        v4i frag = {0, 0, 0, 0};
+        int sq[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (i < nrr_eff) {
+            // i is the same for all lanes of a wave here (a wave covers the 64 pieces of one
+            // rotation when pieces == 64, and whole rotations otherwise), so this branch is uniform
+            const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
+            // this thread's 16 table entries as four 16-byte loads (the table is padded to KS * 32)
+            const uint4 *up4 = (const uint4 *)(upos + k0);
+#pragma unroll
+            for (int w4 = 0; w4 < 4; ++w4) {
+                uint32_t word = 0, live = 0;
+                const uint4 pv = up4[w4];
+                const uint32_t pp[4] = {pv.x, pv.y, pv.z, pv.w};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t k = k0 + w4 * 4 + u;
+                    const uint32_t p = pp[u];
+                    const uint32_t x = (p >> 12) & 0xfff, y = p & 0xfff;
+                    const float *ch = s_img + (p >> 24) * CH;
+                    float val;
+                    if (i) val = bilinear_lds(ch, W, src_c, lim, cs, sn, __fsub_rn((float)x, dst_c), __fsub_rn((float)y, dst_c));
+                    else val = resize_lds(ch, W, I, D, x, y);
+                    word |= quantise_u8(val) << (8 * u);
+                    live |= (k < Ku ? 0xffu : 0u) << (8 * u);
+                }
+                // q - 128 as a signed byte is q ^ 0x80; bytes beyond the union stay 0
+                const int sw = (int)((word ^ 0x80808080u) & live);
+                frag[w4] = sw;
+                if (all_sym) sq[0] = __builtin_amdgcn_sdot4(sw, sw, sq[0], false);
+                else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const uint32_t k = k0 + w4 * 4 + u;
+                        const int v = (int)(signed char)(sw >> (8 * u));
+                        const uint32_t mk = kmask[min(k, Ku - 1)];
+#pragma unroll
+                        for (int s = 0; s < 8; ++s) sq[s] += (mk >> s) & 1 ? v * v : 0;
+                    }
+                }
+            }
+        }
+        Pb[((size_t)b * RTP + rt) * UNIT_V + (piece >> 1) * 64 + g + 32 * (piece & 1)] = frag;
+        if (all_sym) {
+            if (sq[0]) atomicAdd(&s_nb[g][0], sq[0]);
+        } else {
+#pragma unroll
+            for (int s = 0; s < 8; ++s) if (sq[s]) atomicAdd(&s_nb[g][s], sq[s]);
+        }
+    }
+    __syncthreads();
+    {
+        // norm entries of the unit, [symmetry][row]: (15 - j) - 16 |row|^2 with j the accumulator
+        // index the distance kernel's lanes hold this row in (see there).  Rows beyond the last base
+        // rotation get a norm no real distance reaches: they never win the argmin.
+        const uint32_t s = threadIdx.x >> 5, g = threadIdx.x & 31;
+        const int norm = rt * 32 + g < nrr_eff ? (all_sym ? s_nb[g][0] : s_nb[g][s]) : (1 << 26);
+        const int j = 4 * (g >> 3) + (g & 3);
+        int *entries = (int *)(Pb + ((size_t)b * RTP + rt) * UNIT_V + KS * 64);
+        entries[s * 32 + g] = (15 - j) - 16 * norm;
+    }
+}
+
+// Distance + argmin.  A wave keeps its 64 SOM-side rows (8 neurons x 8 symmetries = 2 column
+// tiles) for the WHOLE k range in registers (2 * KS fragments in the accumulation half of the
+// register file, which the MFMA reads directly), so the SOM operand is read once per kernel.
+// The image operand arrives in units of one row tile (32 base rotations, all k, then the tile's
+// 8 x 32 norm entries) and goes through three LDS buffers: unit u is multiplied from buffer
+// u % 3 while unit u+1 moves from the staging registers into the next buffer and the loads of unit
+// u+2 are issued into those registers.  One barrier per unit, in the middle of its k loop, is all
+// the synchronisation: the MFMA stream runs on across unit boundaries.
+// Base rotations are the MFMA's row operand: after the k loop a lane holds, for each of its 2
+// columns (one neuron, one symmetry), 16 base rotations of the tile; their running argmin is
+// kept in-lane by vector-ALU work slotted between the MFMAs of the next unit (from a second
+// accumulator set); per image there is one exchange between the half-waves and three among the 8
+// symmetry lanes.  Every (image, neuron) key is produced by exactly one wave: plain stores, no atomics.
+template <int KS>
+__global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restrict__ Pa, const int *__restrict__ na,
+                                                             const v4i *__restrict__ Pb,
+                                                             unsigned long long *__restrict__ key, uint32_t N,
+                                                             uint32_t B, uint32_t num_rot, uint32_t use_flip,
+                                                             uint32_t RTP, uint32_t groups)
+{
+    constexpr int FRAG_V = KS * 64;                        // 16-byte vectors of fragments per unit
+    constexpr int UNIT_V = FRAG_V + 64;                    // ... plus 8 x 32 norm entries (in memory)
+    constexpr int PER_T = KS / 4;                          // fragment vectors per thread
+    constexpr int H = KS / 2, W0 = KS / 4;                 // k-steps of the barrier / the first LDS store
+    extern __shared__ v4i s_b[];                           // 3 x FRAG_V
+    __shared__ int s_n[4][256];                            // norm entries of units u % 4: [symmetry][row]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t col = lane & 31, half = lane >> 5;
+    const uint32_t slice = blockIdx.x / groups, grp = blockIdx.x % groups;
+    const uint32_t ct0 = (slice * 4 + wave) * 2;           // first of this wave's two column tiles
+    const uint32_t nrr = num_rot / 4;
+    const uint32_t sym = col & 7;                          // same for both column tiles
+
+    // SOM-side fragments for the whole k range, and the row norms of this lane's two columns
+    v4i a[2][KS];
+    int na_l[2];
+    uint32_t n_l[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) a[ct][ks] = Pa[((size_t)(ct0 + ct) * KS + ks) * 64 + lane];
+        na_l[ct] = na[(ct0 + ct) * 32 + col];
+        n_l[ct] = ((ct0 + ct) * 32 + col) >> 3;
+    }
+    // pin the fragments to accumulation registers for the whole kernel: without this the compiler
+    // prefers to re-load them from memory for every row tile
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(a[ct][ks]));
+    const bool sym_ok = (num_rot != 1 || (sym & 3) == 0) && (use_flip || (sym & 4) == 0);
+
+    // The block's units: u -> image grp + (u / RTP) * groups, tile u % RTP.
+    const uint32_t my_images = grp < B ? (B - grp + groups - 1) / groups : 0;
+    const uint32_t nunits = my_images * RTP;
+    if (nunits == 0) return;
+    // source of the next unit to load, advanced without divisions
+    const v4i *src = Pb + (size_t)grp * RTP * UNIT_V + tid;
+    const size_t image_stride = (size_t)groups * RTP * UNIT_V;
+    uint32_t src_rt = 0, src_u = 0;
+    auto advance_src = [&]() {
+        ++src_u;
+        if (++src_rt == RTP) { src_rt = 0; src += image_stride - (size_t)(RTP - 1) * UNIT_V; }
+        else src += UNIT_V;
+    };
+    v4i stage[PER_T];
+    int stage_n;
+    // unit 0 -> buffer 0, unit 1 -> staging registers
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) stage[i] = src[256 * i];
+    stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) s_b[tid + 256 * i] = stage[i];
+    s_n[0][tid] = stage_n;
+    if (nunits > 1) advance_src();
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) stage[i] = src[256 * i];
+    stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+    if (nunits > 2) advance_src();
+    __syncthreads();
+
+    // maximum over the 16 lanes that hold one neuron: the 8 symmetry lanes (two quad exchanges and
+    // a mirror of the half row, all in the data-parallel path) and the other half-wave
+    auto max16 = [&](int v) -> int {
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));    // lane ^ 1
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));    // lane ^ 2
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));   // 7 - lane in the half row
+        return max(v, __shfl_xor(v, 32, 64));
+    };
+
+    // Bookkeeping.  The unit's norm entry of row j of this lane is  cj = (15 - j) - 16 |b_row|^2, so
+    //   cand = 32 acc_j + cj = 16 (|a|^2 - ssd_j) + (15 - j)       (|a|^2 = this column's norm)
+    // and the running signed maximum `m` of cand over rows and tiles is the minimum distance with
+    // the lowest row on ties; `m_rt` remembers the tile that set it (tiles ascend, a later tile
+    // must be strictly better).  16 ssd < 2^30 (checked on the host); rows beyond the last base
+    // rotation carry |b|^2 = 2^26 and never win.
+    int m[2] = {INT_MIN, INT_MIN};
+    uint32_t m_rt[2] = {0, 0};
+    auto finish_image = [&](uint32_t b) {
+        // lexicographic minimum of (distance, variant) over the neuron's 16 lanes in two passes
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+            const uint32_t j = 15u - ((uint32_t)m[ct] & 15u);
+            const int ssd = na_l[ct] - (m[ct] >> 4);
+            const uint32_t i = m_rt[ct] * 32 + 8 * (j >> 2) + 4 * half + (j & 3);
+            const uint32_t k = (sym >> 2) * num_rot + (sym & 3) * nrr + i;
+            const int sv = sym_ok ? -ssd : INT_MIN;
+            const int smax = max16(sv);
+            const int kmax = max16(sv == smax ? -(int)k : INT_MIN);
+            if (half == 0 && sym == 0 && n_l[ct] < N)
+                key[(size_t)b * N + n_l[ct]] = ((unsigned long long)(uint32_t)(-smax) << 16) | (uint32_t)(-kmax);
+            m[ct] = INT_MIN;
+        }
+    };
+    // this lane's 16 norm entries of unit u: rows 8g + 4*half .. +3, g = 0..3
+    auto read_cj = [&](uint32_t u, int (&cj)[16]) {
+        const v4i *nbt = (const v4i *)(&s_n[u & 3][sym * 32 + 4 * half]);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const v4i t = nbt[2 * g];
+            cj[4 * g + 0] = t[0]; cj[4 * g + 1] = t[1]; cj[4 * g + 2] = t[2]; cj[4 * g + 3] = t[3];
+        }
+    };
+
+    // LDS offsets (in vectors) of the buffers holding units u, u+1, u+2
+    uint32_t off_cur = 0, off_next = FRAG_V, off_free = 2 * FRAG_V;
+    v4i bf[4];
+#pragma unroll
+    for (int ks = 0; ks < 3 && ks < KS; ++ks) bf[ks] = s_b[ks * 64 + lane];
+
+    // One unit, hand-scheduled per k-step (nothing crosses the scheduling barriers): the LDS read
+    // of the fragment three k-steps ahead (running on into the next unit's buffer), two MFMAs of
+    // unit u into `acc`, and a slice of the other work: one (column, row) pair of unit u-1's
+    // bookkeeping from `acc_prev` / `cj_prev`, the staging registers (unit u+1) to the next buffer,
+    // the barrier, the loads of unit u+2, and this unit's own norm entries for the next round.
+    auto run_unit = [&](uint32_t u, v16i (&acc)[2][2], int (&cj)[16], const v16i (&acc_prev)[2][2], const int (&cj_prev)[16]) {
+        const v4i *cur = s_b + off_cur + lane, *nxt = s_b + off_next + lane;
+        v4i *dst = s_b + off_next + tid;
+        const int m_before[2] = {m[0], m[1]};
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        auto book = [&](int t0, int t1) {
+#pragma unroll
+            for (int t = t0; t < t1; ++t) {
+                const int ct = (t >> 2) & 1, j = 4 * (t >> 3) + (t & 3);
+                m[ct] = max(m[ct], (int)(((uint32_t)(acc_prev[ct][0][j] + acc_prev[ct][1][j]) << 5) + (uint32_t)cj_prev[j]));
+            }
+            asm volatile("" : "+v"(m[0]), "+v"(m[1]));      // pins the slice where it stands
+        };
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks == H) {
+                // every wave has stored its part of unit u+1 (k-steps W0 .. H-1): wait for this wave's
+                // LDS operations, then meet the others
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+            bf[(ks + 3) & 3] = ks + 3 < KS ? cur[(ks + 3) * 64] : nxt[(ks + 3 - KS) * 64];
+            acc[0][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[0][ks], ks > 1 ? acc[0][ks & 1] : zero, 0, 0, 0);
+            book((2 * ks) * 16 / KS, (2 * ks + 1) * 16 / KS);
+            __builtin_amdgcn_sched_barrier(0);
+            acc[1][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[1][ks], ks > 1 ? acc[1][ks & 1] : zero, 0, 0, 0);
+            book((2 * ks + 1) * 16 / KS, (2 * ks + 2) * 16 / KS);
+            // (past the last unit the staging moves data nobody reads: no branches in the k loop)
+            if (ks >= W0 && ks < W0 + PER_T) dst[256 * (ks - W0)] = stage[ks - W0];
+            if (ks == W0) s_n[(u + 1) & 3][tid] = stage_n;
+            if (ks >= H && ks < H + PER_T) stage[ks - H] = src[256 * (ks - H)];
+            if (ks == H) stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+            if (ks == KS - 2) read_cj(u, cj);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (src_u + 1 < nunits) advance_src();
+        if (u > 0) {
+            const uint32_t rt = (u - 1) % RTP;
+            if (m[0] != m_before[0]) m_rt[0] = rt;
+            if (m[1] != m_before[1]) m_rt[1] = rt;
+            if (rt + 1 == RTP) finish_image(grp + ((u - 1) / RTP) * groups);
+        } else {
+            m[0] = m[1] = INT_MIN;                           // there was no unit before the first
+        }
+        const uint32_t o = off_cur;
+        off_cur = off_next; off_next = off_free; off_free = o;
+    };
+
+    // two accumulator sets (units alternate), each two columns x two chains (even / odd k-steps):
+    // four independent MFMA chains keep the matrix pipe at its issue rate
+    v16i acc0[2][2], acc1[2][2];
+    int cj0[16], cj1[16];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc1[ct][0][j] = acc1[ct][1][j] = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) cj1[j] = 0;
+    for (uint32_t u = 0; u < nunits; u += 2) {
+        run_unit(u, acc0, cj0, acc1, cj1);
+        if (u + 1 < nunits) run_unit(u + 1, acc1, cj1, acc0, cj0);
+    }
+    {
+        // the last unit's bookkeeping
+        const uint32_t u = nunits - 1, rt = u % RTP;
+        const int m_before[2] = {m[0], m[1]};
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct) {
+                const int av = (u & 1) ? acc1[ct][0][j] + acc1[ct][1][j] : acc0[ct][0][j] + acc0[ct][1][j];
+                const int cv = (u & 1) ? cj1[j] : cj0[j];
+                m[ct] = max(m[ct], (int)(((uint32_t)av << 5) + (uint32_t)cv));
+            }
+        if (m[0] != m_before[0]) m_rt[0] = rt;
+        if (m[1] != m_before[1]) m_rt[1] = rt;
+        finish_image(grp + (u / RTP) * groups);              // units end with the last tile of an image
+    }
+}
+
+template <int KS>
+hipError_t launch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool configure_only)
+{
+    const int lds = 3 * KS * 64 * 16;
+    if (configure_only)
+        return hipFuncSetAttribute((const void *)k_dist_mfma_sym_u8<KS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipLaunchKernelGGL((k_dist_mfma_sym_u8<KS>), dim3(g.slices * g.groups), dim3(256), lds, stream, (const v4i *)g.Pa, g.na,
+                       (const v4i *)g.Pb, g.key, g.N, g.B, g.num_rot, g.use_flip, g.RTP, g.groups);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool configure_only)
+{
+    switch (g.KS) {
+    case 8: return launch_dist<8>(stream, g, configure_only);
+    case 16: return launch_dist<16>(stream, g, configure_only);
+    case 24: return launch_dist<24>(stream, g, configure_only);
+    case 32: return launch_dist<32>(stream, g, configure_only);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+namespace pink_sym {
+
+size_t unit_bytes(uint32_t KS) { return ((size_t)KS * 64 + 64) * 16; }
+
+hipError_t pack_som(hipStream_t stream, const float *som, const uint32_t *aoff, signed char *Pa, int *na, uint32_t N,
+                    uint32_t S, uint32_t KS, uint32_t rows)
+{
+    hipLaunchKernelGGL(k_pack_som_sym_u8, dim3(rows), dim3(256), 0, stream, som, aoff, Pa, na, N, S, KS);
+    return hipGetLastError();
+}
+
+hipError_t configure(uint32_t KS, size_t lds_image_bytes)
+{
+    hipError_t e = hipFuncSetAttribute((const void *)k_rotpack_sym_u8, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_image_bytes);
+    if (e != hipSuccess) return e;
+    DistArgs g{};
+    g.KS = KS;
+    return dispatch_dist(nullptr, g, true);
+}
+
+hipError_t rotpack(hipStream_t stream, const RotpackArgs &g)
+{
+    const size_t lds = (size_t)g.C * (g.I + 1) * (g.I + 1) * sizeof(float);
+    const uint32_t blocks = ((g.B + 7) / 8) * 8 * g.RTP;              // 8 images per span of ids, see the kernel
+    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(blocks), dim3(256), lds, stream, g.images, (v4i *)g.Pb, g.cos_t, g.sin_t, g.upos,
+                       g.kmask, g.Ku, g.all_sym, g.C, g.I, g.nrr_eff, g.D, g.KS, g.RTP, g.B);
+    return hipGetLastError();
+}
+
+hipError_t dist(hipStream_t stream, const DistArgs &g) { return dispatch_dist(stream, g, false); }
+
+}  // namespace pink_sym

@@ -28,6 +28,7 @@
 #include <type_traits>
 #include <vector>
 
+#include "mfma_u8_sym.h"
 #include "pink_hip.h"
 
 namespace {
@@ -652,7 +653,6 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
     }
 }
 
-#include "mfma_u8_sym.inc"
 #include "mfma_int_gemm.inc"
 
 // ---------------------------------------------------------------------------------
@@ -927,9 +927,9 @@ int run_pack_som(pink_hip_ctx *ctx)
         return launch_check(ctx, "k_pack_planes");
     }
     if (ctx->mfma_sym) {
-        hipLaunchKernelGGL(k_pack_som_sym_u8, dim3(ctx->slices * 8 * 32), dim3(256), 0, ctx->stream, ctx->d_som,
-                           ctx->d_aoff, ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->KSs);
-        return launch_check(ctx, "k_pack_som_sym_u8");
+        HIP_TRY(ctx, pink_sym::pack_som(ctx->stream, ctx->d_som, ctx->d_aoff, ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->KSs,
+                                        ctx->slices * 8 * 32));
+        return PINK_HIP_OK;
     }
     if (ctx->mfma) {
         hipLaunchKernelGGL(k_pack_som_u8, dim3(ctx->NT * 32), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
@@ -1233,8 +1233,7 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipMemcpy(ctx->d_upos, upos.data(), upos.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             HIP_TRY(ctx, hipMemcpy(ctx->d_aoff, aoff.data(), aoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             HIP_TRY(ctx, hipMemcpy(ctx->d_kmask, kmask.data(), kmask.size(), hipMemcpyHostToDevice));
-            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotpack_sym_u8, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (int)lds_img));
+            HIP_TRY(ctx, pink_sym::configure(ctx->KSs, lds_img));
         }
     }
     if (ctx->mfma) {
@@ -1302,7 +1301,7 @@ int init_ctx(pink_hip_ctx *ctx)
     if (ctx->gemm)
         per_image = (size_t)ctx->R * ctx->S * 4 + (size_t)(c.ed_type == PINK_HIP_UINT16 ? 2 : 1) * (ctx->Rp / 32) * ctx->gKS * 1024 +
                     (size_t)ctx->Rp * 8 + (size_t)ctx->N * 24;
-    if (ctx->mfma_sym) per_image = (size_t)ctx->RTP * ctx->KSs * 1024 + (size_t)ctx->RTP * 32 * 8 * 4 + (size_t)ctx->N * 24;
+    if (ctx->mfma_sym) per_image = (size_t)ctx->RTP * pink_sym::unit_bytes(ctx->KSs) + (size_t)ctx->N * 24;
     if (ctx->trainer) {
         // images whose variants are prepared ahead of the sequential distance/update chain
         size_t b = c.max_batch ? c.max_batch : 64;
@@ -1327,8 +1326,7 @@ int init_ctx(pink_hip_ctx *ctx)
     if (ctx->mfma_sym) {
         TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->slices * 8 * ctx->KSs * 1024));
         TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->slices * 8 * 32));
-        TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RTP * ctx->KSs * 1024));
-        TRY(dev_alloc(ctx, &ctx->d_nb, B * ctx->RTP * 32 * 8));
+        TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RTP * pink_sym::unit_bytes(ctx->KSs)));
     } else if (ctx->gemm) {
         const size_t planes = c.ed_type == PINK_HIP_UINT16 ? 2 : 1;
         const size_t a_vec = planes * (ctx->Np / 32) * ctx->gKS * 64, b_vec = planes * (ctx->Rp / 32) * ctx->gKS * 64;
@@ -1409,33 +1407,23 @@ int run_dist_mfma(pink_hip_ctx *ctx, uint32_t B)
 int run_rotpack_sym(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
     Timed t(ctx, kClsRotate);
-    const size_t lds = (size_t)ctx->C * (ctx->I + 1) * (ctx->I + 1) * sizeof(float);
-    const uint32_t blocks = ((B + 7) / 8) * 8 * ctx->RTP;          // 8 images per span of ids, see the kernel
-    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(blocks), dim3(256), lds, ctx->stream, dev_images, (v4i *)ctx->d_Pb,
-                       ctx->d_nb, ctx->d_cos, ctx->d_sin, ctx->d_upos, ctx->d_kmask, ctx->Ku, ctx->all_sym, ctx->C,
-                       ctx->I, ctx->nrr_eff, ctx->D, ctx->KSs, ctx->RTP, B);
-    return launch_check(ctx, "k_rotpack_sym_u8");
-}
-
-template <int KS>
-void launch_dist_sym(pink_hip_ctx *ctx, uint32_t B)
-{
-    const uint32_t groups = std::min(ctx->groups, B);
-    hipLaunchKernelGGL((k_dist_mfma_sym_u8<KS>), dim3(ctx->slices * groups), dim3(256), 0, ctx->stream,
-                       (const v4i *)ctx->d_Pa, ctx->d_na, (const v4i *)ctx->d_Pb, ctx->d_nb, ctx->d_key, ctx->N, B,
-                       ctx->cfg.num_rot, ctx->cfg.use_flip, ctx->nrr_eff, ctx->RTP, groups);
+    pink_sym::RotpackArgs g{};
+    g.images = dev_images; g.Pb = ctx->d_Pb; g.cos_t = ctx->d_cos; g.sin_t = ctx->d_sin; g.upos = ctx->d_upos;
+    g.kmask = ctx->d_kmask; g.Ku = ctx->Ku; g.all_sym = ctx->all_sym; g.C = ctx->C; g.I = ctx->I; g.nrr_eff = ctx->nrr_eff;
+    g.D = ctx->D; g.KS = ctx->KSs; g.RTP = ctx->RTP; g.B = B;
+    HIP_TRY(ctx, pink_sym::rotpack(ctx->stream, g));
+    return PINK_HIP_OK;
 }
 
 int run_dist_sym(pink_hip_ctx *ctx, uint32_t B)
 {
     Timed t(ctx, kClsDist);
-    switch (ctx->KSs) {
-    case 8: launch_dist_sym<8>(ctx, B); break;
-    case 16: launch_dist_sym<16>(ctx, B); break;
-    case 24: launch_dist_sym<24>(ctx, B); break;
-    default: launch_dist_sym<32>(ctx, B); break;
-    }
-    return launch_check(ctx, "k_dist_mfma_sym_u8");
+    pink_sym::DistArgs g{};
+    g.Pa = ctx->d_Pa; g.na = ctx->d_na; g.Pb = ctx->d_Pb; g.key = ctx->d_key; g.N = ctx->N; g.B = B;
+    g.num_rot = ctx->cfg.num_rot; g.use_flip = ctx->cfg.use_flip; g.RTP = ctx->RTP; g.KS = ctx->KSs;
+    g.slices = ctx->slices; g.groups = std::min(ctx->groups, B);
+    HIP_TRY(ctx, pink_sym::dist(ctx->stream, g));
+    return PINK_HIP_OK;
 }
 
 int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
