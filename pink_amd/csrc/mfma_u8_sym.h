@@ -10,9 +10,15 @@
 
 namespace pink_sym {
 
-// Once per context: allow the rotation kernel its LDS image (C x (I+1) x (I+1) floats) and the
-// distance kernel of this KS (8, 16, 24 or 32 k-steps) its three LDS buffers.
-hipError_t configure(uint32_t KS, size_t lds_image_bytes);
+// Once per context: allow the rotation kernel its LDS images (C x (I+1) x (I+1) floats each) and
+// the distance kernel of this KS (8, 16, 24 or 32 k-steps) its three LDS buffers.
+hipError_t configure(uint32_t KS, uint32_t C, uint32_t I);
+
+// The geometry of the base rotations (source offset and bilinear weights per rotation and union
+// position), built once per context into `table` (rot_table_bytes() bytes of device memory).
+size_t rot_table_bytes(uint32_t KS, uint32_t RTP);
+hipError_t build_rot_table(hipStream_t stream, const float *cos_t, const float *sin_t, const uint32_t *upos, uint32_t Ku,
+                           uint32_t I, uint32_t D, uint32_t nrr_eff, uint32_t KS, uint32_t RTP, void *table);
 
 // Bytes of one unit of the image operand: one row tile of 32 base rotations = KS fragments of
 // 1 KiB, followed by 1 KiB of norm entries [8 symmetries][32 rows].
@@ -25,10 +31,10 @@ hipError_t pack_som(hipStream_t stream, const float *som, const uint32_t *aoff, 
 struct RotpackArgs {
     const float *images;        // B x C x I x I
     void *Pb;                   // B x RTP units
-    const float *cos_t, *sin_t;
-    const uint32_t *upos;
+    const uint32_t *tab_idx;    // table built by build_rot_table: offsets ...
+    const void *tab_w;          // ... and weights
     const unsigned char *kmask;
-    uint32_t Ku, all_sym, C, I, nrr_eff, D, KS, RTP, B;
+    uint32_t Ku, all_sym, C, I, nrr_eff, KS, RTP, B;
 };
 hipError_t rotpack(hipStream_t stream, const RotpackArgs &args);
 

@@ -70,159 +70,237 @@ __global__ __launch_bounds__(256) void k_pack_som_sym_u8(const float *__restrict
     if (threadIdx.x == 0) na[m] = s_sum[0];
 }
 
-// Image operand: base rotations only.  A block handles one row tile (32 base rotations) of one
-// image.  The image is staged in LDS with one extra zero column per row and one extra zero row per
-// channel, so the two neighbours that the bilinear rule reads with weight 0 at the last
-// row / column (ImageProcessingLib/rotate.h:50,62-63) need no index clamp.  A thread evaluates
-// 16 consecutive union positions of one rotation (bilinear in the CPU's operation order,
-// quantised, shifted), stores them as one 16-byte piece of a fragment, and adds their squares
-// to the 8 per-symmetry norms of that rotation according to kmask (bit s of kmask[k] set when
-// union position k belongs to P_s).
-//   upos[k] = (channel << 24 | x << 12 | y) of union element k, k < Ku (0 beyond, up to KS * 32).
-// Bilinear value of base rotation i > 0 at the neuron pixel whose centred coordinates are
-// (px, py) = (x - (D-1)/2, y - (D-1)/2), from the padded LDS image.  Branch-free: the taps are
-// read at the clamped position and the result is replaced by 0 when the source position lies
-// outside the image (ImageProcessingLib/rotate.h:40-44), so a wave never diverges here.
-__device__ __forceinline__ float bilinear_lds(const float *__restrict__ s_img, uint32_t W, float src_c, float lim,
-                                              float cs, float sn, float px, float py)
+// Image operand: base rotations only.
+//
+// Where a rotated pixel comes from does not depend on the image: for base rotation i and union
+// position k the bilinear rule of ImageProcessingLib/rotate.h:31-65 reads four neighbours at a
+// fixed place of the source image with fixed weights.  k_rot_table evaluates that geometry once
+// per context, in the CPU's operation order:
+//   tab_idx(i, k) = offset of the upper-left neighbour in the padded LDS image (channel included),
+//   tab_w(i, k)   = (cx*cy, cx*ry, rx*cy, rx*ry), the four products the CPU forms first.
+// Where the source position lies outside the image (value 0, rotate.h:40-44) or k is beyond the
+// union, the entry points at a zero cell of the padding with four zero weights: 0 for finite pixels.
+// Base rotation 0 is the centre crop / pad of ImageProcessingLib/resize.h:15-40: weight 1 on the
+// copied pixel, 0 on the others (1*x + 0 + 0 + 0 == x for the finite inputs the quantisation is
+// defined for).  The per-image work that is left is four products, three sums and the quantisation.
+//   upos[k] = (channel << 24 | x << 12 | y) of union element k, k < Ku.
+__global__ __launch_bounds__(256) void k_rot_table(const float *__restrict__ cos_t, const float *__restrict__ sin_t,
+                                                   const uint32_t *__restrict__ upos, uint32_t Ku, uint32_t I,
+                                                   uint32_t D, uint32_t nrr_eff, uint32_t Kp, uint32_t rows,
+                                                   uint32_t *__restrict__ tab_idx, float4 *__restrict__ tab_w)
 {
-    const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
-    const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
-    const bool outside = sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim;
-    const float sxc = __builtin_amdgcn_fmed3f(sxf, 0.0f, lim), syc = __builtin_amdgcn_fmed3f(syf, 0.0f, lim);
-    const uint32_t ix = (uint32_t)sxc, iy = (uint32_t)syc;
-    const float rx = __fsub_rn(sxc, (float)ix), ry = __fsub_rn(syc, (float)iy);
-    const float cx = __fsub_rn(1.0f, rx), cy = __fsub_rn(1.0f, ry);
-    const float *t = s_img + ix * W + iy;
-    const float a = __fmul_rn(__fmul_rn(cx, cy), t[0]);
-    const float b = __fmul_rn(__fmul_rn(cx, ry), t[1]);
-    const float c = __fmul_rn(__fmul_rn(rx, cy), t[W]);
-    const float d = __fmul_rn(__fmul_rn(rx, ry), t[W + 1]);
-    const float v = __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
-    return outside ? 0.0f : v;
-}
-
-// Centre crop / centre pad (base rotation 0), ImageProcessingLib/resize.h:15-40.
-__device__ __forceinline__ float resize_lds(const float *__restrict__ s_img, uint32_t W, uint32_t I, uint32_t D,
-                                            uint32_t x, uint32_t y)
-{
-    if (I >= D) {
-        const uint32_t m = (I - D) / 2;
-        return s_img[(x + m) * W + (y + m)];
+    const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= rows * Kp) return;
+    const uint32_t i = t / Kp, k = t % Kp;
+    const uint32_t W = I + 1, CH = W * W;
+    uint32_t idx = I;                                     // row 0 of the extra column: 0.0
+    float4 w = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (i < nrr_eff && k < Ku) {
+        const uint32_t p = upos[k];
+        const uint32_t c = p >> 24, x = (p >> 12) & 0xfff, y = p & 0xfff;
+        if (i == 0) {
+            if (I >= D) {
+                const uint32_t m = (I - D) / 2;
+                idx = c * CH + (x + m) * W + (y + m);
+                w.x = 1.0f;
+            } else {
+                const uint32_t m = (D - I) / 2;
+                const uint32_t sx = x - m, sy = y - m;     // wraps below the margin: caught by the range test
+                if (sx < I && sy < I) { idx = c * CH + sx * W + sy; w.x = 1.0f; }
+            }
+        } else {
+            const float cs = cos_t[i], sn = sin_t[i];
+            const float src_c = __fmul_rn((float)(I - 1), 0.5f), dst_c = __fmul_rn((float)(D - 1), 0.5f);
+            const float lim = (float)(I - 1);
+            const float px = __fsub_rn((float)x, dst_c), py = __fsub_rn((float)y, dst_c);
+            const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+            const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+            if (!(sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim)) {
+                // the neighbours one past the last row / column carry weight 0 and exist in the
+                // padded LDS image (rotate.h:50,62-63 reads them out of bounds)
+                const uint32_t ix = (uint32_t)sxf, iy = (uint32_t)syf;
+                const float rx = __fsub_rn(sxf, (float)ix), ry = __fsub_rn(syf, (float)iy);
+                const float cx = __fsub_rn(1.0f, rx), cy = __fsub_rn(1.0f, ry);
+                idx = c * CH + ix * W + iy;
+                w.x = __fmul_rn(cx, cy); w.y = __fmul_rn(cx, ry); w.z = __fmul_rn(rx, cy); w.w = __fmul_rn(rx, ry);
+            }
+        }
     }
-    const uint32_t m = (D - I) / 2;
-    const uint32_t sx = x - m, sy = y - m;
-    return (sx < I && sy < I) ? s_img[sx * W + sy] : 0.0f;
+    // piece-interleaved so that the 64 lanes of a wave, which hold 64 consecutive pieces of a
+    // rotation, read consecutive 16-byte entries: weights [i][j][piece], offsets [i][j / 4][piece][j % 4]
+    const uint32_t pieces = Kp / 16, piece = k / 16, j = k % 16;
+    tab_w[((size_t)i * 16 + j) * pieces + piece] = w;
+    tab_idx[(((size_t)i * 4 + j / 4) * pieces + piece) * 4 + j % 4] = idx;
 }
 
-// q = uint8(x * 255) saturated (NaN -> 0): multiply, clamp (v_med3_f32), convert.
-__device__ __forceinline__ uint32_t quantise_u8(float x)
+// Byte `byte` of `word` = q = uint8(x * 255), truncated and saturated to [0, 255] (NaN -> 0):
+// multiply, truncate, then the saturating convert-and-pack (which alone would round to nearest).
+__device__ __forceinline__ uint32_t pack_quantised_u8(float x, uint32_t byte, uint32_t word)
 {
-    return (uint32_t)__builtin_amdgcn_fmed3f(__fmul_rn(x, 255.0f), 0.0f, 255.0f);
+    return __builtin_amdgcn_cvt_pk_u8_f32(__builtin_truncf(__fmul_rn(x, 255.0f)), byte, word);
 }
 
-__global__ __launch_bounds__(256) void k_rotpack_sym_u8(const float *__restrict__ images, v4i *__restrict__ Pb,
-                                                        const float *__restrict__ cos_t,
-                                                        const float *__restrict__ sin_t,
-                                                        const uint32_t *__restrict__ upos,
+// A block handles one row tile (32 base rotations) of G images, which it keeps in LDS with one
+// extra zero column per row and one extra zero row per channel.  A thread evaluates 16
+// consecutive union positions of one rotation for every image -- a table entry is read once and
+// applied G times --, stores them as one 16-byte piece of a fragment per image, and adds their
+// squares to the 8 per-symmetry norms of that rotation according to kmask (bit s of kmask[k] set
+// when union position k belongs to P_s).
+template <int G>
+__global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict__ images, v4i *__restrict__ Pb,
+                                                        const uint32_t *__restrict__ tab_idx,
+                                                        const float4 *__restrict__ tab_w,
                                                         const unsigned char *__restrict__ kmask, uint32_t Ku,
                                                         uint32_t all_sym, uint32_t C, uint32_t I, uint32_t nrr_eff,
-                                                        uint32_t D, uint32_t KS, uint32_t RTP, uint32_t B)
+                                                        uint32_t KS, uint32_t RTP, uint32_t B)
 {
-    extern __shared__ float s_img[];                      // C x (I + 1) x (I + 1), zero padded
+    extern __shared__ float s_img[];                      // G x C x (I + 1) x (I + 1), zero padded
+    __shared__ int s_nb[G][32][8];
     const uint32_t UNIT_V = KS * 64 + 64;                 // 16-byte vectors per unit: fragments, then norm entries
-    __shared__ int s_nb[32][8];
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The
-    // id is decoded so that all blocks of one image share id % 8, i.e. one XCD: the image then
-    // leaves HBM once instead of once per XCD.
+    // id is decoded so that all blocks of one group of images share id % 8, i.e. one XCD: the
+    // images then leave HBM once instead of once per XCD.
     const uint32_t lin = blockIdx.x;
-    const uint32_t span = 8 * RTP;                        // ids covering 8 images
+    const uint32_t span = 8 * RTP;                        // ids covering 8 groups
     const uint32_t rt = (lin % span) / 8;
-    const uint32_t b = (lin / span) * 8 + (lin % 8);
-    if (b >= B) return;
-    const uint32_t W = I + 1, CH = W * W, II = I * I;
-    const float *img = images + (size_t)b * C * II;
-    s_nb[threadIdx.x >> 3][threadIdx.x & 7] = 0;
-    for (uint32_t c = 0; c < C; ++c) {
-        // coalesced copy of the I x I channel into the padded tile; (r, q) advance without divisions
-        uint32_t r = threadIdx.x / I, q = threadIdx.x % I;
-        for (uint32_t t = threadIdx.x; t < II; t += 256) {
-            s_img[c * CH + r * W + q] = img[(size_t)c * II + t];
-            q += 256;
-            while (q >= I) { q -= I; ++r; }
+    const uint32_t b0 = ((lin / span) * 8 + (lin % 8)) * G;
+    if (b0 >= B) return;
+    const uint32_t ng = min((uint32_t)G, B - b0);
+    const uint32_t W = I + 1, CH = W * W, II = I * I, IMG = C * CH;
+    const uint32_t nthreads = blockDim.x;
+    for (uint32_t t = threadIdx.x; t < G * 32 * 8; t += nthreads) (&s_nb[0][0][0])[t] = 0;
+    // Copy the batch into the padded tiles.  The loads of up to 8 elements per thread are issued
+    // before the first is used, so the block pays the memory latency once, not once per image.
+    {
+        const float *src = images + (size_t)b0 * C * II;
+        const uint32_t total = ng * C * II;
+        if ((I & 3) == 0) {
+            // rows are whole float4s: 16-byte loads, one division per vector
+            const float4 *src4 = (const float4 *)src;
+            const uint32_t total4 = total / 4;
+            for (uint32_t base = 0; base < total4; base += 8 * nthreads) {
+                float4 v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t e = base + j * nthreads + threadIdx.x;
+                    if (e < total4) v[j] = src4[e];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t e = base + j * nthreads + threadIdx.x;
+                    if (e < total4) {
+                        const uint32_t gc = (4 * e) / II, rem = (4 * e) % II;
+                        float *d = s_img + gc * CH + (rem / I) * W + rem % I;
+                        d[0] = v[j].x; d[1] = v[j].y; d[2] = v[j].z; d[3] = v[j].w;
+                    }
+                }
+            }
+        } else {
+            for (uint32_t base = 0; base < total; base += 8 * nthreads) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t e = base + j * nthreads + threadIdx.x;
+                    if (e < total) v[j] = src[e];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t e = base + j * nthreads + threadIdx.x;
+                    if (e < total) {
+                        const uint32_t gc = e / II, rem = e % II;
+                        s_img[gc * CH + (rem / I) * W + rem % I] = v[j];
+                    }
+                }
+            }
         }
-        for (uint32_t t = threadIdx.x; t <= I; t += 256) {
-            s_img[c * CH + t * W + I] = 0.0f;             // extra column
-            s_img[c * CH + I * W + t] = 0.0f;             // extra row
+        for (uint32_t t = threadIdx.x; t < ng * C * W; t += nthreads) {
+            const uint32_t gc = t / W, r = t % W;
+            s_img[gc * CH + r * W + I] = 0.0f;            // extra column
+            s_img[gc * CH + I * W + r] = 0.0f;            // extra row
         }
     }
     __syncthreads();
 
-    const float src_c = __fmul_rn((float)(I - 1), 0.5f), dst_c = __fmul_rn((float)(D - 1), 0.5f);
-    const float lim = (float)(I - 1);
     const uint32_t pieces = KS * 2;                       // 16-element pieces per row
     for (uint32_t t = threadIdx.x; t < 32 * pieces; t += blockDim.x) {
         const uint32_t g = t / pieces, piece = t % pieces;
         const uint32_t i = rt * 32 + g;                   // base rotation
         const uint32_t k0 = piece * 16;
-        v4i frag = {0, 0, 0, 0};
-        int sq[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        uint32_t word[G][4];
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+            for (int w4 = 0; w4 < 4; ++w4) word[gi][w4] = 0;
+        uint32_t live[4] = {0, 0, 0, 0};
         if (i < nrr_eff) {
-            // i is the same for all lanes of a wave here (a wave covers the 64 pieces of one
-            // rotation when pieces == 64, and whole rotations otherwise), so this branch is uniform
-            const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
-            // this thread's 16 table entries as four 16-byte loads (the table is padded to KS * 32)
-            const uint4 *up4 = (const uint4 *)(upos + k0);
+            // (uniform per wave: a wave covers the pieces of whole rotations)
+            const uint4 *ti = (const uint4 *)tab_idx + (size_t)i * 4 * pieces + piece;
+            const float4 *tw = tab_w + (size_t)i * 16 * pieces + piece;
 #pragma unroll
             for (int w4 = 0; w4 < 4; ++w4) {
-                uint32_t word = 0, live = 0;
-                const uint4 pv = up4[w4];
-                const uint32_t pp[4] = {pv.x, pv.y, pv.z, pv.w};
+                const uint4 iv = ti[w4 * pieces];
+                const uint32_t ii[4] = {iv.x, iv.y, iv.z, iv.w};
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const uint32_t k = k0 + w4 * 4 + u;
-                    const uint32_t p = pp[u];
-                    const uint32_t x = (p >> 12) & 0xfff, y = p & 0xfff;
-                    const float *ch = s_img + (p >> 24) * CH;
-                    float val;
-                    if (i) val = bilinear_lds(ch, W, src_c, lim, cs, sn, __fsub_rn((float)x, dst_c), __fsub_rn((float)y, dst_c));
-                    else val = resize_lds(ch, W, I, D, x, y);
-                    word |= quantise_u8(val) << (8 * u);
-                    live |= (k < Ku ? 0xffu : 0u) << (8 * u);
-                }
-                // q - 128 as a signed byte is q ^ 0x80; bytes beyond the union stay 0
-                const int sw = (int)((word ^ 0x80808080u) & live);
-                frag[w4] = sw;
-                if (all_sym) sq[0] = __builtin_amdgcn_sdot4(sw, sw, sq[0], false);
-                else {
+                    const float4 wv = tw[(4 * w4 + u) * pieces];
+                    const float *tap = s_img + ii[u];
+                    live[w4] |= (k0 + 4 * w4 + u < Ku ? 0xffu : 0u) << (8 * u);
+                    // (all G images, also past the end of the batch: what is computed from LDS nobody
+                    // filled is dropped below, and the loop stays free of branches)
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const uint32_t k = k0 + w4 * 4 + u;
-                        const int v = (int)(signed char)(sw >> (8 * u));
-                        const uint32_t mk = kmask[min(k, Ku - 1)];
-#pragma unroll
-                        for (int s = 0; s < 8; ++s) sq[s] += (mk >> s) & 1 ? v * v : 0;
+                    for (int gi = 0; gi < G; ++gi) {
+                        const float *tp = tap + gi * IMG;
+                        const float a = __fmul_rn(wv.x, tp[0]);
+                        const float b = __fmul_rn(wv.y, tp[1]);
+                        const float c = __fmul_rn(wv.z, tp[W]);
+                        const float d = __fmul_rn(wv.w, tp[W + 1]);
+                        const float v = __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
+                        word[gi][w4] = pack_quantised_u8(v, u, word[gi][w4]);
                     }
                 }
             }
         }
-        Pb[((size_t)b * RTP + rt) * UNIT_V + (piece >> 1) * 64 + g + 32 * (piece & 1)] = frag;
-        if (all_sym) {
-            if (sq[0]) atomicAdd(&s_nb[g][0], sq[0]);
-        } else {
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (sq[s]) atomicAdd(&s_nb[g][s], sq[s]);
+        for (int gi = 0; gi < G; ++gi) {
+            if (gi < (int)ng) {
+                v4i frag;
+                int sq[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int w4 = 0; w4 < 4; ++w4) {
+                    // q - 128 as a signed byte is q ^ 0x80; bytes beyond the union stay 0
+                    const int sw = (int)((word[gi][w4] ^ 0x80808080u) & live[w4]);
+                    frag[w4] = sw;
+                    if (all_sym) sq[0] = __builtin_amdgcn_sdot4(sw, sw, sq[0], false);
+                    else {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const uint32_t k = k0 + w4 * 4 + u;
+                            const int v = (int)(signed char)(sw >> (8 * u));
+                            const uint32_t mk = kmask[min(k, Ku - 1)];
+#pragma unroll
+                            for (int s = 0; s < 8; ++s) sq[s] += (mk >> s) & 1 ? v * v : 0;
+                        }
+                    }
+                }
+                Pb[((size_t)(b0 + gi) * RTP + rt) * UNIT_V + (piece >> 1) * 64 + g + 32 * (piece & 1)] = frag;
+                if (all_sym) {
+                    if (sq[0]) atomicAdd(&s_nb[gi][g][0], sq[0]);
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 8; ++s) if (sq[s]) atomicAdd(&s_nb[gi][g][s], sq[s]);
+                }
+            }
         }
     }
     __syncthreads();
-    {
+    for (uint32_t gi = 0; gi < ng && threadIdx.x < 256; ++gi) {
         // norm entries of the unit, [symmetry][row]: (15 - j) - 16 |row|^2 with j the accumulator
         // index the distance kernel's lanes hold this row in (see there).  Rows beyond the last base
         // rotation get a norm no real distance reaches: they never win the argmin.
         const uint32_t s = threadIdx.x >> 5, g = threadIdx.x & 31;
-        const int norm = rt * 32 + g < nrr_eff ? (all_sym ? s_nb[g][0] : s_nb[g][s]) : (1 << 26);
+        const int norm = rt * 32 + g < nrr_eff ? (all_sym ? s_nb[gi][g][0] : s_nb[gi][g][s]) : (1 << 26);
         const int j = 4 * (g >> 3) + (g & 3);
-        int *entries = (int *)(Pb + ((size_t)b * RTP + rt) * UNIT_V + KS * 64);
+        int *entries = (int *)(Pb + ((size_t)(b0 + gi) * RTP + rt) * UNIT_V + KS * 64);
         entries[s * 32 + g] = (15 - j) - 16 * norm;
     }
 }
@@ -476,23 +554,61 @@ hipError_t pack_som(hipStream_t stream, const float *som, const uint32_t *aoff, 
     return hipGetLastError();
 }
 
-hipError_t configure(uint32_t KS, size_t lds_image_bytes)
+// images per block of the rotation kernel: as many as let two blocks share a CU's LDS (one loads
+// its images while the other computes), next to their norm counters
+uint32_t images_per_block(size_t lds_image_bytes)
 {
-    hipError_t e = hipFuncSetAttribute((const void *)k_rotpack_sym_u8, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_image_bytes);
+    const size_t budget = 72 * 1024;
+    return lds_image_bytes * 4 <= budget ? 4 : lds_image_bytes * 2 <= budget ? 2 : 1;
+}
+
+template <int G>
+hipError_t launch_rotpack(hipStream_t stream, const RotpackArgs &g, bool configure_only)
+{
+    const size_t lds = (size_t)G * g.C * (g.I + 1) * (g.I + 1) * sizeof(float);
+    if (configure_only)
+        return hipFuncSetAttribute((const void *)k_rotpack_sym_u8<G>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    const uint32_t groups = (g.B + G - 1) / G;
+    const uint32_t blocks = ((groups + 7) / 8) * 8 * g.RTP;           // 8 groups per span of ids, see the kernel
+    hipLaunchKernelGGL(k_rotpack_sym_u8<G>, dim3(blocks), dim3(G >= 4 ? 512 : 256), lds, stream, g.images, (v4i *)g.Pb, g.tab_idx,
+                       (const float4 *)g.tab_w, g.kmask, g.Ku, g.all_sym, g.C, g.I, g.nrr_eff, g.KS, g.RTP, g.B);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_rotpack(hipStream_t stream, const RotpackArgs &g, bool configure_only)
+{
+    switch (images_per_block((size_t)g.C * (g.I + 1) * (g.I + 1) * sizeof(float))) {
+    case 4: return launch_rotpack<4>(stream, g, configure_only);
+    case 2: return launch_rotpack<2>(stream, g, configure_only);
+    default: return launch_rotpack<1>(stream, g, configure_only);
+    }
+}
+
+hipError_t configure(uint32_t KS, uint32_t C, uint32_t I)
+{
+    RotpackArgs r{};
+    r.C = C; r.I = I;
+    hipError_t e = dispatch_rotpack(nullptr, r, true);
     if (e != hipSuccess) return e;
     DistArgs g{};
     g.KS = KS;
     return dispatch_dist(nullptr, g, true);
 }
 
-hipError_t rotpack(hipStream_t stream, const RotpackArgs &g)
+size_t rot_table_bytes(uint32_t KS, uint32_t RTP) { return (size_t)RTP * 32 * KS * 32 * (sizeof(uint32_t) + sizeof(float4)); }
+
+hipError_t build_rot_table(hipStream_t stream, const float *cos_t, const float *sin_t, const uint32_t *upos, uint32_t Ku,
+                           uint32_t I, uint32_t D, uint32_t nrr_eff, uint32_t KS, uint32_t RTP, void *table)
 {
-    const size_t lds = (size_t)g.C * (g.I + 1) * (g.I + 1) * sizeof(float);
-    const uint32_t blocks = ((g.B + 7) / 8) * 8 * g.RTP;              // 8 images per span of ids, see the kernel
-    hipLaunchKernelGGL(k_rotpack_sym_u8, dim3(blocks), dim3(256), lds, stream, g.images, (v4i *)g.Pb, g.cos_t, g.sin_t, g.upos,
-                       g.kmask, g.Ku, g.all_sym, g.C, g.I, g.nrr_eff, g.D, g.KS, g.RTP, g.B);
+    const uint32_t rows = RTP * 32, Kp = KS * 32;
+    float4 *tab_w = (float4 *)table;                                   // weights first: 16-byte aligned
+    uint32_t *tab_idx = (uint32_t *)(tab_w + (size_t)rows * Kp);
+    hipLaunchKernelGGL(k_rot_table, dim3((rows * Kp + 255) / 256), dim3(256), 0, stream, cos_t, sin_t, upos, Ku, I, D, nrr_eff,
+                       Kp, rows, tab_idx, tab_w);
     return hipGetLastError();
 }
+
+hipError_t rotpack(hipStream_t stream, const RotpackArgs &g) { return dispatch_rotpack(stream, g, false); }
 
 hipError_t dist(hipStream_t stream, const DistArgs &g) { return dispatch_dist(stream, g, false); }
 

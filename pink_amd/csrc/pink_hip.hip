@@ -776,6 +776,7 @@ struct pink_hip_ctx {
     size_t lds_dist = 0, lds_rotpack = 0;
     int num_cu = 256;
     signed char *d_Pa = nullptr, *d_Pb = nullptr;
+    void *d_rtab = nullptr;                // geometry table of the base rotations (symmetric MFMA path)
     int *d_na = nullptr, *d_nb = nullptr;
     unsigned short *d_poff = nullptr;
     uint32_t *d_need = nullptr;
@@ -1097,7 +1098,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -1233,7 +1234,11 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipMemcpy(ctx->d_upos, upos.data(), upos.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             HIP_TRY(ctx, hipMemcpy(ctx->d_aoff, aoff.data(), aoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             HIP_TRY(ctx, hipMemcpy(ctx->d_kmask, kmask.data(), kmask.size(), hipMemcpyHostToDevice));
-            HIP_TRY(ctx, pink_sym::configure(ctx->KSs, lds_img));
+            HIP_TRY(ctx, pink_sym::configure(ctx->KSs, ctx->C, ctx->I));
+            HIP_TRY(ctx, hipMalloc(&ctx->d_rtab, pink_sym::rot_table_bytes(ctx->KSs, ctx->RTP)));
+            HIP_TRY(ctx, pink_sym::build_rot_table(ctx->stream, ctx->d_cos, ctx->d_sin, ctx->d_upos, ctx->Ku, ctx->I, ctx->D,
+                                                   ctx->nrr_eff, ctx->KSs, ctx->RTP, ctx->d_rtab));
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
         }
     }
     if (ctx->mfma) {
@@ -1408,9 +1413,11 @@ int run_rotpack_sym(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
     Timed t(ctx, kClsRotate);
     pink_sym::RotpackArgs g{};
-    g.images = dev_images; g.Pb = ctx->d_Pb; g.cos_t = ctx->d_cos; g.sin_t = ctx->d_sin; g.upos = ctx->d_upos;
+    const size_t entries = (size_t)ctx->RTP * 32 * ctx->KSs * 32;
+    g.images = dev_images; g.Pb = ctx->d_Pb; g.tab_w = ctx->d_rtab;
+    g.tab_idx = (const uint32_t *)((const char *)ctx->d_rtab + entries * 16);
     g.kmask = ctx->d_kmask; g.Ku = ctx->Ku; g.all_sym = ctx->all_sym; g.C = ctx->C; g.I = ctx->I; g.nrr_eff = ctx->nrr_eff;
-    g.D = ctx->D; g.KS = ctx->KSs; g.RTP = ctx->RTP; g.B = B;
+    g.KS = ctx->KSs; g.RTP = ctx->RTP; g.B = B;
     HIP_TRY(ctx, pink_sym::rotpack(ctx->stream, g));
     return PINK_HIP_OK;
 }
