@@ -55,6 +55,18 @@ __device__ __forceinline__ unsigned long long wave_min_u64(unsigned long long v)
     return v;
 }
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// q = T(x * factor) truncated, saturated to [0, factor] (CudaLib/copy_and_transform_kernel.h:27-28)
+__device__ __forceinline__ int32_t quantise(float x, float factor)
+{
+    const float v = __fmul_rn(x, factor);
+    if (!(v > 0.0f)) return 0;
+    if (v >= factor) return (int32_t)factor;
+    return (int32_t)v;
+}
+
 // Value of base rotation `i` (angle i * 2pi / num_rot, 0 <= angle < 90 degrees) of one
 // channel at neuron pixel (x, y).  i == 0 is the centre crop / centre pad of
 // ImageProcessingLib/resize.h:15-40; i > 0 is ImageProcessingLib/rotate.h:31-65 with
@@ -106,13 +118,29 @@ __device__ __forceinline__ float base_pixel(const float *__restrict__ img, uint3
 // flip (ImageProcessingLib/flip.h:14-30): F[x][y] = V[D-1-x][y].
 // Block (0, 0, b) also resets the image's argmin keys.
 // ---------------------------------------------------------------------------------
+// Operand packing fused into the rotation kernel (blocks that hold their base rotation in LDS):
+// the region of every variant goes straight from LDS into the distance kernel's operand, so the
+// variants are not read back.  symoff[sym * Epad + e] = channel << 24 | position in the base
+// rotation of region element e under symmetry sym = flip * 4 + quarter.
+//   PACK 1: float32 rows, opnd[(b * Rpad + k) * Epad + e]            (k = variant index)
+//   PACK 2 / 3: uint8 / uint16 byte planes in MFMA fragment order (see mfma_int_gemm.inc) and
+//               the row norms |V|^2; single channel only.
+struct PackArgs {
+    const uint32_t *symoff;
+    void *opnd;            // float rows, or byte planes
+    long long *norm;       // integer modes: [b][Rp]
+    uint32_t E, Epad, rows_pad, KS;
+};
+
+template <int PACK>
 __global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
-                                                uint32_t use_flip, uint32_t use_lds)
+                                                uint32_t use_flip, uint32_t use_lds, PackArgs pk)
 {
     extern __shared__ float s_base[];
+    __shared__ unsigned long long s_norm[8];
     const uint32_t i = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
     const uint32_t nrr = num_rot / 4;
     const uint32_t R = num_rot * (use_flip ? 2u : 1u);
@@ -124,6 +152,7 @@ __global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images
 
     if (i == 0 && c == 0)
         for (uint32_t n = threadIdx.x; n < N; n += blockDim.x) key[(size_t)b * N + n] = ~0ull;
+    if (PACK >= 2 && threadIdx.x < 8) s_norm[threadIdx.x] = 0;
 
     if (use_lds) {
         for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x)
@@ -144,6 +173,69 @@ __global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images
                     const uint32_t k = f * num_rot + q * nrr + i;
                     out[((size_t)k * C + c) * DD + p] = s_base[a * D + bb];
                 }
+            }
+        }
+        if constexpr (PACK == 1) {
+            float *opnd = (float *)pk.opnd + (size_t)b * pk.rows_pad * pk.Epad;
+            for (uint32_t f = 0; f < nf; ++f)
+                for (uint32_t q = 0; q < nq; ++q) {
+                    const uint32_t *so = pk.symoff + (size_t)(f * 4 + q) * pk.Epad;
+                    float *row = opnd + (size_t)(f * num_rot + q * nrr + i) * pk.Epad;
+                    for (uint32_t e = threadIdx.x; e < pk.E; e += blockDim.x) {
+                        const uint32_t po = so[e];
+                        if ((po >> 24) == c) row[e] = s_base[po & 0xffffffu];
+                    }
+                }
+        } else if constexpr (PACK >= 2) {
+            constexpr bool U16 = PACK == 3;
+            constexpr uint32_t planes = U16 ? 2 : 1;
+            const float factor = U16 ? 65535.0f : 255.0f;
+            const size_t plane_stride = (size_t)(pk.rows_pad / 32) * pk.KS * 64;
+            v4i *P = (v4i *)pk.opnd + (size_t)b * planes * plane_stride;
+            for (uint32_t f = 0; f < nf; ++f)
+                for (uint32_t q = 0; q < nq; ++q) {
+                    const uint32_t sym = f * 4 + q, r = f * num_rot + q * nrr + i;
+                    const uint32_t *so = pk.symoff + (size_t)sym * pk.Epad;
+                    long long sq = 0;
+                    for (uint32_t piece = threadIdx.x; piece < pk.KS * 2; piece += blockDim.x) {
+                        v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+                        const uint4 *so4 = (const uint4 *)(so + piece * 16);
+#pragma unroll
+                        for (int w4 = 0; w4 < 4; ++w4) {
+                            const uint4 pv = so4[w4];
+                            const uint32_t pp[4] = {pv.x, pv.y, pv.z, pv.w};
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                if (piece * 16 + w4 * 4 + u < pk.E) {
+                                    const int qv = quantise(s_base[pp[u] & 0xffffffu], factor);
+                                    int h, l = 0;
+                                    if (U16) {
+                                        const int cv = qv - 32768;
+                                        h = cv >> 8;
+                                        l = (cv & 255) - 128;
+                                    } else {
+                                        h = qv - 128;
+                                    }
+                                    const long long v = U16 ? 256 * h + l : h;
+                                    sq += v * v;
+                                    hi[w4] |= (h & 255) << (8 * u);
+                                    lo[w4] |= (l & 255) << (8 * u);
+                                }
+                            }
+                        }
+                        const size_t frag = ((size_t)(r >> 5) * pk.KS + (piece >> 1)) * 64 + (r & 31) + 32 * (piece & 1);
+                        P[frag] = hi;
+                        if (U16) P[plane_stride + frag] = lo;
+                    }
+#pragma unroll
+                    for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
+                    if ((threadIdx.x & 63) == 0) atomicAdd(&s_norm[sym], (unsigned long long)sq);
+                }
+            __syncthreads();
+            if (threadIdx.x < 8) {
+                const uint32_t f = threadIdx.x >> 2, q = threadIdx.x & 3;
+                if (f < nf && q < nq)
+                    pk.norm[(size_t)b * pk.rows_pad + f * num_rot + q * nrr + i] = (long long)s_norm[threadIdx.x];
             }
         }
     } else {
@@ -177,13 +269,6 @@ __global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images
 // conv: float32 copy, or quantisation q = T(x * factor) saturated to [0, factor]
 // (CudaLib/copy_and_transform_kernel.h:27-28) held as int32.
 // ---------------------------------------------------------------------------------
-__device__ __forceinline__ int32_t quantise(float x, float factor)
-{
-    const float v = __fmul_rn(x, factor);
-    if (!(v > 0.0f)) return 0;
-    if (v >= factor) return (int32_t)factor;
-    return (int32_t)v;
-}
 
 template <bool QUANT>
 __global__ __launch_bounds__(256) void k_pack_som(const float *__restrict__ som, const uint32_t *__restrict__ off,
@@ -472,8 +557,6 @@ __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict
 // k = flip * num_rot + quarter * (num_rot / 4) + i travels in the argmin key, so ties
 // still resolve to the lowest variant index.
 // ---------------------------------------------------------------------------------
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 // Rotation + quantisation + packing, no float variants written.  Block (tile, b): base
 // rotations 4*tile .. 4*tile+3 of image b are evaluated only at the pixels some region
@@ -777,6 +860,8 @@ struct pink_hip_ctx {
     int num_cu = 256;
     signed char *d_Pa = nullptr, *d_Pb = nullptr;
     void *d_rtab = nullptr;                // geometry table of the base rotations (symmetric MFMA path)
+    uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
+    bool fused_pack = false;
     int *d_na = nullptr, *d_nb = nullptr;
     unsigned short *d_poff = nullptr;
     uint32_t *d_need = nullptr;
@@ -953,14 +1038,37 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
     const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->D * sizeof(float) : 0;
-    hipLaunchKernelGGL(k_rotate, grid, dim3(256), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin,
-                       ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,
-                       ctx->use_lds ? 1u : 0u);
+    PackArgs pk{};
+    int pack = 0;
+    if (ctx->fused_pack) {
+        pk.symoff = ctx->d_symoff;
+        pk.E = ctx->E;
+        pk.Epad = ctx->Epad;
+        if (ctx->gemm) {
+            pack = ctx->cfg.ed_type == PINK_HIP_UINT16 ? 3 : 2;
+            pk.opnd = ctx->d_gPb; pk.norm = ctx->d_gnb; pk.rows_pad = ctx->Rp; pk.KS = ctx->gKS;
+        } else {
+            pack = 1;
+            pk.opnd = ctx->d_rotT; pk.rows_pad = ctx->Rpad;
+        }
+    }
+#define LAUNCH_ROTATE(P_)                                                                                          \
+    hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(256), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
+                       ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
+                       ctx->use_lds ? 1u : 0u, pk)
+    switch (pack) {
+    case 1: LAUNCH_ROTATE(1); break;
+    case 2: LAUNCH_ROTATE(2); break;
+    case 3: LAUNCH_ROTATE(3); break;
+    default: LAUNCH_ROTATE(0); break;
+    }
+#undef LAUNCH_ROTATE
     return launch_check(ctx, "k_rotate");
 }
 
 int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 {
+    if (ctx->fused_pack) return PINK_HIP_OK;              // k_rotate wrote the operand already
     Timed t(ctx, kClsPack);
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
@@ -1098,7 +1206,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff};
     for (void *p : bufs) if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -1353,6 +1461,35 @@ int init_ctx(pink_hip_ctx *ctx)
     } else {
         TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad));
         TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
+        // rows beyond R and elements beyond the region must read as zero whoever fills the rest
+        HIP_TRY(ctx, hipMemset(ctx->d_rotT, 0, B * ctx->Epad * ctx->Rpad * sizeof(uint32_t)));
+    }
+    // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
+    // integer contexts, whenever the kernel keeps its base rotation in LDS.
+    ctx->fused_pack = ctx->use_lds && !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && ctx->D <= 4096 &&
+                      (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
+    if (ctx->fused_pack) {
+        const uint32_t D = ctx->D, DD = D * D;
+        std::vector<uint32_t> symoff((size_t)8 * ctx->Epad, 0u);
+        for (uint32_t sym = 0; sym < 8; ++sym) {
+            const uint32_t f = sym >> 2, q = sym & 3;
+            for (uint32_t e = 0; e < ctx->E; ++e) {
+                // variant pixel (x, y) of symmetry (f, q) is base-rotation pixel (a, bb): the flip
+                // reverses the rows of the quarter turn (see k_rotate)
+                const uint32_t ch = region[e] / DD, x = (region[e] % DD) / D, y = region[e] % D;
+                const uint32_t xs = f ? D - 1 - x : x;
+                uint32_t a, bb;
+                switch (q) {
+                case 0: a = xs; bb = y; break;
+                case 1: a = D - 1 - y; bb = xs; break;
+                case 2: a = D - 1 - xs; bb = D - 1 - y; break;
+                default: a = y; bb = D - 1 - xs; break;
+                }
+                symoff[(size_t)sym * ctx->Epad + e] = (ch << 24) | (a * D + bb);
+            }
+        }
+        TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
+        HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, symoff.data(), symoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
     }
     TRY(dev_alloc(ctx, &ctx->d_bmu_scratch, 1));
     TRY(dev_alloc(ctx, &ctx->d_dist, B * ctx->N));
