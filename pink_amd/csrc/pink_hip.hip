@@ -745,12 +745,22 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
 //   w = w - ((w - x) * f),  f = factors[bmu * N + n], skipped when f == 0,
 // and refreshes the region elements of the packed distance operand in the same pass.
 // ---------------------------------------------------------------------------------
+// Operand refresh of the integer GEMM path inside the update: the byte planes of the updated
+// elements (fragment order of mfma_int_gemm.inc) and the row norm |V|^2, accumulated per block
+// into `na_next` (zeroed by the distance kernel's finish step, which read the other buffer).
+struct UpdatePlanes {
+    signed char *Pa;            // null: not this path
+    long long *na_next;
+    const long long *na_cur;
+    uint32_t KS, Np, u16;
+};
+
 __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const float *__restrict__ rot,
                                                 const unsigned long long *__restrict__ key,
                                                 const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
                                                 uint32_t N, uint32_t S, uint32_t parts, uint32_t shift,
                                                 void *__restrict__ somP, const uint32_t *__restrict__ inv,
-                                                uint32_t Epad, float qfactor)
+                                                uint32_t Epad, float qfactor, UpdatePlanes up)
 {
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
@@ -777,12 +787,18 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     if (n == 0 && part == 0 && tid == 0) *bmu_out = bmu;
 
     const float f = factors[(size_t)bmu * N + n];
-    if (f == 0.0f) return;
+    if (f == 0.0f) {
+        // untouched neuron: its operand row stands, its norm moves to the next buffer
+        if (up.Pa && part == 0 && tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], (unsigned long long)up.na_cur[n]);
+        return;
+    }
     const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
     const float *__restrict__ x = rot + (size_t)r * S;
     float *__restrict__ w = som + (size_t)n * S;
     const uint32_t chunk = (S + parts - 1) / parts;
     const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
+    long long sq = 0;
+    const size_t plane_bytes = (size_t)(up.Np / 32) * up.KS * 64 * 16;
     for (uint32_t j = j0 + tid; j < j1; j += 256) {
         const float wv = w[j];
         const float nv = __fsub_rn(wv, __fmul_rn(__fsub_rn(wv, x[j]), f));
@@ -792,10 +808,37 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         if (inv) {
             const uint32_t k = inv[j];
             if (k != 0xffffffffu) {
-                if (qfactor > 0.0f) ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
-                else ((float *)somP)[(size_t)n * Epad + k] = nv;
+                if (up.Pa) {
+                    const int q = quantise(nv, qfactor);
+                    const size_t byte = ((((size_t)(n >> 5) * up.KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
+                    if (up.u16) {
+                        const int c = q - 32768;
+                        const int h = c >> 8, l = (c & 255) - 128;
+                        up.Pa[byte] = (signed char)h;
+                        up.Pa[plane_bytes + byte] = (signed char)l;
+                        const long long v = 256 * h + l;
+                        sq += v * v;
+                    } else {
+                        const int h = q - 128;
+                        up.Pa[byte] = (signed char)h;
+                        sq += h * h;
+                    }
+                } else if (qfactor > 0.0f) {
+                    ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
+                } else {
+                    ((float *)somP)[(size_t)n * Epad + k] = nv;
+                }
             }
         }
+    }
+    if (up.Pa) {
+        // (f depends on the block only, so every thread of the block is here)
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
+        __syncthreads();                                   // s_val was last read as s_idx[0]'s partner above
+        if ((tid & 63) == 0) s_val[tid >> 6] = (unsigned long long)sq;
+        __syncthreads();
+        if (tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], s_val[0] + s_val[1] + s_val[2] + s_val[3]);
     }
 }
 
@@ -862,6 +905,8 @@ struct pink_hip_ctx {
     void *d_rtab = nullptr;                // geometry table of the base rotations (symmetric MFMA path)
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
+    bool fused_som = false;                // integer GEMM trainer: k_update refreshes the SOM planes and norms itself
+    uint32_t na_cur = 0;                   // which half of d_gna holds the norms of the current SOM operand
     int *d_na = nullptr, *d_nb = nullptr;
     unsigned short *d_poff = nullptr;
     uint32_t *d_need = nullptr;
@@ -1006,10 +1051,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
             hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(1024), 2 * ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
         else
             hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(1024), ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
         return launch_check(ctx, "k_pack_planes");
     }
     if (ctx->mfma_sym) {
@@ -1151,7 +1196,8 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot)
                        (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ctx->gks_per, ctx->gslices, tiles_per_xcd);
     const uint32_t rows_per_chunk = 32;
     hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
-                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, ctx->d_gna, ctx->d_gnb + (size_t)slot * ctx->Rp,
+                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np,
+                       ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np, ctx->d_gnb + (size_t)slot * ctx->Rp,
                        ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Np, ctx->R, ctx->Rp, ctx->gslices, rows_per_chunk);
 }
 
@@ -1180,10 +1226,19 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     Timed t(ctx, kClsUpdate);
     uint32_t parts = (1024 + ctx->N - 1) / ctx->N;
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
+    UpdatePlanes up{};
+    if (ctx->fused_som) {
+        up.Pa = (signed char *)ctx->d_gPa;
+        up.na_cur = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np;
+        up.na_next = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
+        up.KS = ctx->gKS; up.Np = ctx->Np; up.u16 = ctx->cfg.ed_type == PINK_HIP_UINT16;
+    }
     hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
-                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP, ctx->gemm ? nullptr : ctx->d_inv, ctx->Epad,
-                       is_int(ctx) ? (float)ctx->factor : 0.0f);
+                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,
+                       (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,
+                       is_int(ctx) ? (float)ctx->factor : 0.0f, up);
+    if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
 }
 
@@ -1446,7 +1501,7 @@ int init_ctx(pink_hip_ctx *ctx)
         const size_t dot_n = ctx->gslices * planes * (size_t)ctx->Rp * ctx->Np;   // int32 (uint8) or int64 (uint16) per element
         TRY(dev_alloc(ctx, &ctx->d_gPa, a_vec));
         TRY(dev_alloc(ctx, &ctx->d_gPb, B * b_vec));
-        TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)ctx->Np));
+        TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)2 * ctx->Np));   // two halves, see na_cur
         TRY(dev_alloc(ctx, &ctx->d_gnb, B * ctx->Rp));
         TRY(dev_alloc(ctx, &ctx->d_dot, dot_n));
         // rows beyond N / R and elements beyond the region are never written: they must read as zero
@@ -1506,6 +1561,7 @@ int init_ctx(pink_hip_ctx *ctx)
         if (one_to_one) {
             TRY(dev_alloc(ctx, &ctx->d_inv, inv.size()));
             HIP_TRY(ctx, hipMemcpy(ctx->d_inv, inv.data(), inv.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+            ctx->fused_som = ctx->gemm;
         }
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
@@ -1702,7 +1758,7 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
         for (uint32_t b = 0; b < B; ++b) {
             TRY(run_dist(ctx, b, 1));
             TRY(run_update(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
-            if (!ctx->d_inv || ctx->gemm) TRY(run_pack_som(ctx));
+            if (!ctx->d_inv || (ctx->gemm && !ctx->fused_som)) TRY(run_pack_som(ctx));
         }
     }
     return PINK_HIP_OK;
