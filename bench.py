@@ -41,8 +41,8 @@ MEASURED_FMA_NOPACK_TFLOPS = 72.5
 # HBM bytes per image from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/cfg1_map_u8_hbm_traffic.txt),
 # scaled by the same counters' readings for a 256 MiB device-to-device copy (FETCH x2.0, WRITE x1.0).
 MEASURED_TRAFFIC_PER_IMAGE = {
-    ("cfg1", 3, "rotate"): 17.0e3 + 108.9e3,
-    ("cfg1", 3, "distance"): 108.1e3 + 0.8e3,
+    ("cfg1", 3, "rotate"): 57.8e3 + 138.1e3,     # image + part of the geometry table read; units written
+    ("cfg1", 3, "distance"): 108.1e3 + 0.8e3,    # units read once; keys written
 }
 
 
@@ -57,8 +57,8 @@ def algorithmic_per_image(w, E, path):
     rot_bytes = R * S * 4 + w.image_size * 4              # all variants written once, image read once
     if path == 2:      # uint8 MFMA, symmetries on the image side: ceil(nrr/4) tiles of 32 rows + norms
         rot_bytes = w.image_size * 4 + -(-nrr // 4) * 32 * (kp + 4)
-    elif path == 3:    # uint8 MFMA, symmetries on the SOM side: ceil(nrr/32) tiles of 32 rows + 8 norms per row
-        rot_bytes = w.image_size * 4 + -(-nrr // 32) * 32 * (kp + 32)
+    elif path == 3:    # uint8 MFMA, symmetries on the SOM side: ceil(nrr/32) units of 32 rows + 1 KiB of norm entries
+        rot_bytes = w.image_size * 4 + -(-nrr // 32) * (32 * kp + 1024)
     return {
         "rotate": {"bytes": rot_bytes},
         # region of every variant read as float32 and written in the distance type
