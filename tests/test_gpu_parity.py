@@ -209,6 +209,84 @@ def test_map_parity(name, n, ed_type, choice):
     assert np.array_equal(best, obest)
 
 
+SYM_SHAPES = [
+    # N, C, I, D, nrot, flip, ed, shape, images   -- each exercises another corner of the resident-SOM kernels
+    (3, 1, 24, 18, 40, True, 16, capi.QUADRATIC, 5),       # 8 k-steps, one unit per image, one column tile, batch not a multiple of 4
+    (70, 1, 32, 24, 160, True, 22, capi.QUADRATIC, 9),     # 16 k-steps, two units per image, three SOM slices
+    (150, 1, 45, 32, 360, True, 27, capi.QUADRATIC, 3),    # 24 k-steps, three units, five slices, image edge not a multiple of 4
+    (33, 1, 40, 44, 360, False, 32, capi.QUADRATIC, 37),   # 32 k-steps, padded neurons (I < D), no flip, more images than one group
+    (20, 2, 20, 16, 8, True, 10, capi.QUADRATIC, 6),       # two channels, two base rotations
+    (12, 1, 16, 12, 4, True, 12, capi.QUADRATIC, 4),       # quarter turns only
+    (12, 1, 16, 12, 1, True, 12, capi.QUADRATIC, 4),       # flip only
+    (25, 1, 40, 29, 16, True, 21, capi.CIRCULAR, 7),       # circular region, odd diameter
+    (1, 1, 28, 28, 360, True, 28, capi.QUADRATIC, 1),      # a single neuron, a single image
+]
+
+
+@pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_,n", SYM_SHAPES)
+def test_map_uint8_kernels_over_shapes(N, C_, I, D, nrot, flip, ed, shape_, n):
+    say("map u8 shapes", N, C_, I, D, nrot, flip, ed, shape_, n)
+    rng = np.random.default_rng(N * 7 + I + nrot)
+    som = rng.random((N, C_ * D * D), dtype=np.float32)
+    imgs = rng.random((n, C_, I, I), dtype=np.float32)
+    R = nrot * (2 if flip else 1)
+    som[N // 2] = O.rotated_images(imgs[0], C_, I, D, nrot, flip)[R - 1].ravel()       # an exact match at the last variant
+    s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, capi.UINT8)
+    oheat, obest = O.map_images(s, som, imgs)
+    ran = []
+    for choice in (capi.KERNEL_AUTO, capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA, capi.KERNEL_MFMA_GEMM):
+        try:
+            ctx = capi.Context(N, C_, I, D, nrot, flip, ed, shape_, capi.UINT8, None, max_batch=16, kernel_choice=choice)
+        except capi.PinkError:
+            assert choice in (capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM)
+            continue
+        with ctx:
+            ran.append(ctx.distance_kernel)
+            ctx.set_som(som)
+            heat, best = ctx.map(imgs)
+            heat_again, best_again = ctx.map(imgs[:1])        # a second, shorter call on the same context
+        assert np.array_equal(bits(heat), bits(oheat)), choice
+        assert np.array_equal(best, obest), choice
+        assert np.array_equal(bits(heat_again), bits(oheat[:1])) and np.array_equal(best_again, obest[:1]), choice
+    say("   kernels that ran:", ran)
+    assert capi.KERNEL_MFMA_GEMM in ran and capi.KERNEL_MFMA_SYM in ran
+
+
+FUSED_TRAIN_SHAPES = [
+    # N, C, I, D, nrot, flip, ed, shape, ed_type, images  -- operand packing inside the rotation and update kernels
+    (10, 1, 20, 16, 24, True, 11, capi.CIRCULAR, capi.UINT16, 5),
+    (70, 1, 20, 14, 8, False, 14, capi.QUADRATIC, capi.UINT8, 6),     # two column tiles, no flip
+    (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.UINT8, 4),        # three channels: packing stays in its own kernel
+    (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.FLOAT, 4),        # three channels, float32 rows from the rotation kernel
+    (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.FLOAT, 3),           # region repeats channel 0 (CPU rule): no inverse table
+    (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.UINT16, 3),
+]
+
+
+@pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_,ed_type,n", FUSED_TRAIN_SHAPES)
+def test_train_over_shapes(N, C_, I, D, nrot, flip, ed, shape_, ed_type, n):
+    say("train shapes", N, C_, I, D, nrot, flip, ed, shape_, ed_type, n)
+    rng = np.random.default_rng(N + I * 3 + nrot)
+    som0 = rng.random((N, C_ * D * D), dtype=np.float32)
+    imgs = rng.random((n, C_, I, I), dtype=np.float32)
+    F = capi.make_update_factors(capi.CARTESIAN, [N], capi.GAUSSIAN, 1.0, 0.5)
+    F[F < 0.01] = 0.0                                        # some neurons are skipped by the update
+    s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, ed_type)
+    want = som0.copy()
+    obmu = O.train(s, want, imgs, F)
+    with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type, F, max_batch=2) as ctx:
+        ctx.set_som(som0)
+        bmu = np.concatenate([ctx.train(imgs[:1]), ctx.train(imgs[1:])])      # two calls, groups of two images
+        som = ctx.get_som()
+        # the packed operand the update kernel maintains must match a fresh pack of the same weights
+        d1, ssd1, best1 = ctx.distance(imgs[0])
+        ctx.set_som(som)
+        d2, ssd2, best2 = ctx.distance(imgs[0])
+    assert np.array_equal(bmu, obmu)
+    assert np.array_equal(bits(som), bits(want))             # gate 1e-4; achieved and asserted: bit-exact
+    assert np.array_equal(bits(d1), bits(d2)) and np.array_equal(ssd1, ssd2) and np.array_equal(best1, best2)
+
+
 def test_reference_mapper_known_answers():
     # test/CudaTest/mapper.cu:115-119 in float, uint8 and uint16; circular_ed.cu:23-53
     for som_dim, nd, idim, ed, nrot, flip in [(1, 2, 2, 2, 1, False), (1, 3, 3, 2, 1, False), (1, 3, 3, 2, 360, False),
