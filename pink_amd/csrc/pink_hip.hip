@@ -903,6 +903,13 @@ struct pink_hip_ctx {
     int num_cu = 256;
     signed char *d_Pa = nullptr, *d_Pb = nullptr;
     void *d_rtab = nullptr;                // geometry table of the base rotations (symmetric MFMA path)
+    // Staging of the host-pointer entry points, kept across calls (the reference's per-image
+    // operator() makes one call per image): device buffers for a chunk of images and their
+    // results, and a pinned bounce buffer through which small transfers go.
+    float *st_img = nullptr, *st_heat = nullptr;
+    uint32_t *st_best = nullptr, *st_bmu = nullptr;
+    size_t st_images = 0;                  // capacity of the staging buffers, in images
+    char *st_pin = nullptr;                // kPinBytes in, kPinBytes out
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
     bool fused_som = false;                // integer GEMM trainer: k_update refreshes the SOM planes and norms itself
@@ -1263,6 +1270,8 @@ int free_all(pink_hip_ctx *ctx)
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
                     ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff};
     for (void *p : bufs) if (p) (void)hipFree(p);
+    for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
+    if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
 }
@@ -1764,6 +1773,44 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
     return PINK_HIP_OK;
 }
 
+constexpr size_t kPinBytes = (size_t)1 << 20;
+
+// Staging for `n` images per chunk (grown on demand, freed with the context).
+int ensure_staging(pink_hip_ctx *ctx, size_t n)
+{
+    if (!ctx->st_pin) {
+        if (hipHostMalloc((void **)&ctx->st_pin, 2 * kPinBytes, hipHostMallocDefault) != hipSuccess) {
+            ctx->st_pin = nullptr;
+            return fail(ctx, PINK_HIP_ENOMEM, "pinned host allocation failed");
+        }
+    }
+    if (n <= ctx->st_images) return PINK_HIP_OK;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu})
+        if (p) (void)hipFree(p);
+    ctx->st_img = ctx->st_heat = nullptr;
+    ctx->st_best = ctx->st_bmu = nullptr;
+    ctx->st_images = 0;
+    hipError_t e = hipMalloc((void **)&ctx->st_img, n * ctx->isz * sizeof(float));
+    if (e == hipSuccess && ctx->trainer) e = hipMalloc((void **)&ctx->st_bmu, n * sizeof(uint32_t));
+    if (e == hipSuccess && !ctx->trainer) e = hipMalloc((void **)&ctx->st_heat, n * ctx->N * sizeof(float));
+    if (e == hipSuccess && !ctx->trainer) e = hipMalloc((void **)&ctx->st_best, n * ctx->N * sizeof(uint32_t));
+    if (e != hipSuccess) return fail(ctx, PINK_HIP_ENOMEM, "staging allocation failed");
+    ctx->st_images = n;
+    return PINK_HIP_OK;
+}
+
+// Host -> device on the context's stream; small transfers go through the pinned buffer (one
+// memcpy on the host, then a true asynchronous copy).
+hipError_t stage_in(pink_hip_ctx *ctx, void *dev, const void *host, size_t bytes)
+{
+    if (bytes <= kPinBytes) {
+        memcpy(ctx->st_pin, host, bytes);
+        return hipMemcpyAsync(dev, ctx->st_pin, bytes, hipMemcpyHostToDevice, ctx->stream);
+    }
+    return hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream);
+}
+
 int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out)
 {
     if (!ctx || (!host_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train: null argument");
@@ -1773,28 +1820,23 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
     // Stage the images in chunks of at most ~1 GiB.
     const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
     const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
-    float *d_img = nullptr;
-    uint32_t *d_bmu = nullptr;
-    HIP_TRY(ctx, hipMalloc((void **)&d_img, chunk * img_bytes));
-    if (hipMalloc((void **)&d_bmu, chunk * sizeof(uint32_t)) != hipSuccess) {
-        (void)hipFree(d_img);
-        return fail(ctx, PINK_HIP_ENOMEM, "pink_hip_train: device allocation failed");
-    }
-    int rc = PINK_HIP_OK;
-    for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += chunk) {
+    TRY(ensure_staging(ctx, chunk));
+    for (uint32_t done = 0; done < n_images; done += chunk) {
         const uint32_t n = std::min(chunk, n_images - done);
-        hipError_t e = hipMemcpyAsync(d_img, host_images + (size_t)done * ctx->isz, n * img_bytes, hipMemcpyHostToDevice,
-                                      ctx->stream);
-        if (e == hipSuccess) rc = pink_hip_train_device(ctx, d_img, n, d_bmu);
-        if (e == hipSuccess && rc == PINK_HIP_OK && host_bmu_out)
-            e = hipMemcpyAsync(host_bmu_out + done, d_bmu, n * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream);
-        if (e == hipSuccess && rc == PINK_HIP_OK) e = hipStreamSynchronize(ctx->stream);
-        if (e != hipSuccess) rc = fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_train: ") + hipGetErrorString(e));
+        HIP_TRY(ctx, stage_in(ctx, ctx->st_img, host_images + (size_t)done * ctx->isz, n * img_bytes));
+        TRY(pink_hip_train_device(ctx, ctx->st_img, n, ctx->st_bmu));
+        if (host_bmu_out) {
+            const size_t out_bytes = n * sizeof(uint32_t);
+            const bool small = out_bytes <= kPinBytes;
+            HIP_TRY(ctx, hipMemcpyAsync(small ? (void *)(ctx->st_pin + kPinBytes) : (void *)(host_bmu_out + done), ctx->st_bmu,
+                                        out_bytes, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+            if (small) memcpy(host_bmu_out + done, ctx->st_pin + kPinBytes, out_bytes);
+        } else {
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));      // the host images are the caller's again on return
+        }
     }
-    (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree(d_img);
-    (void)hipFree(d_bmu);
-    return rc;
+    return PINK_HIP_OK;
 }
 
 int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, float *dev_heatmap_out,
@@ -1821,30 +1863,28 @@ int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
     const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
-    float *d_img = nullptr, *d_heat = nullptr;
-    uint32_t *d_best = nullptr;
-    hipError_t e = hipMalloc((void **)&d_img, chunk * img_bytes);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_heat, (size_t)chunk * ctx->N * sizeof(float));
-    if (e == hipSuccess) e = hipMalloc((void **)&d_best, (size_t)chunk * ctx->N * sizeof(uint32_t));
-    int rc = e == hipSuccess ? PINK_HIP_OK : fail(ctx, PINK_HIP_ENOMEM, "pink_hip_map: device allocation failed");
-    for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += chunk) {
+    TRY(ensure_staging(ctx, chunk));
+    for (uint32_t done = 0; done < n_images; done += chunk) {
         const uint32_t n = std::min(chunk, n_images - done);
-        e = hipMemcpyAsync(d_img, host_images + (size_t)done * ctx->isz, n * img_bytes, hipMemcpyHostToDevice, ctx->stream);
-        if (e == hipSuccess) rc = pink_hip_map_device(ctx, d_img, n, d_heat, d_best);
-        if (e == hipSuccess && rc == PINK_HIP_OK)
-            e = hipMemcpyAsync(host_heatmap_out + (size_t)done * ctx->N, d_heat, (size_t)n * ctx->N * sizeof(float),
-                               hipMemcpyDeviceToHost, ctx->stream);
-        if (e == hipSuccess && rc == PINK_HIP_OK && host_best_rot_out)
-            e = hipMemcpyAsync(host_best_rot_out + (size_t)done * ctx->N, d_best, (size_t)n * ctx->N * sizeof(uint32_t),
-                               hipMemcpyDeviceToHost, ctx->stream);
-        if (e == hipSuccess && rc == PINK_HIP_OK) e = hipStreamSynchronize(ctx->stream);
-        if (e != hipSuccess) rc = fail(ctx, PINK_HIP_EDEVICE, std::string("pink_hip_map: ") + hipGetErrorString(e));
+        HIP_TRY(ctx, stage_in(ctx, ctx->st_img, host_images + (size_t)done * ctx->isz, n * img_bytes));
+        TRY(pink_hip_map_device(ctx, ctx->st_img, n, ctx->st_heat, ctx->st_best));
+        const size_t heat_bytes = (size_t)n * ctx->N * sizeof(float);       // the best rotations take as many bytes
+        const bool small = 2 * heat_bytes <= kPinBytes;
+        char *pin_out = ctx->st_pin + kPinBytes;
+        float *heat_dst = host_heatmap_out + (size_t)done * ctx->N;
+        uint32_t *best_dst = host_best_rot_out ? host_best_rot_out + (size_t)done * ctx->N : nullptr;
+        HIP_TRY(ctx, hipMemcpyAsync(small ? (void *)pin_out : (void *)heat_dst, ctx->st_heat, heat_bytes, hipMemcpyDeviceToHost,
+                                    ctx->stream));
+        if (best_dst)
+            HIP_TRY(ctx, hipMemcpyAsync(small ? (void *)(pin_out + heat_bytes) : (void *)best_dst, ctx->st_best, heat_bytes,
+                                        hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        if (small) {
+            memcpy(heat_dst, pin_out, heat_bytes);
+            if (best_dst) memcpy(best_dst, pin_out + heat_bytes, heat_bytes);
+        }
     }
-    (void)hipStreamSynchronize(ctx->stream);
-    if (d_img) (void)hipFree(d_img);
-    if (d_heat) (void)hipFree(d_heat);
-    if (d_best) (void)hipFree(d_best);
-    return rc;
+    return PINK_HIP_OK;
 }
 
 int pink_hip_rotate(pink_hip_ctx *ctx, const float *host_image, float *host_variants_out)
