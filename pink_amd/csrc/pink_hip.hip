@@ -1199,13 +1199,21 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot)
     const uint32_t planes = U16 ? 2 : 1;
     const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
     const uint32_t tiles_per_xcd = ((ctx->Rp / 64) * (ctx->Np / 64) + 7) / 8;
+    GemmFinish fin{};
+    long long *na = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, *na_other = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
+    const long long *nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
+    unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
+    if (ctx->gslices == 1) {
+        // a block sees the whole k range: it finishes its tile itself
+        fin.key = key; fin.na = na; fin.na_other = na_other; fin.nb = nb; fin.N = ctx->N; fin.R = ctx->R;
+    }
     hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * ctx->gslices), dim3(256), 0, ctx->stream, ctx->d_gPa, pb,
-                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ctx->gks_per, ctx->gslices, tiles_per_xcd);
+                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ctx->gks_per, ctx->gslices, tiles_per_xcd, fin);
+    if (ctx->gslices == 1) return;
     const uint32_t rows_per_chunk = 32;
     hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
-                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np,
-                       ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np, ctx->d_gnb + (size_t)slot * ctx->Rp,
-                       ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Np, ctx->R, ctx->Rp, ctx->gslices, rows_per_chunk);
+                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, na, na_other, nb, key, ctx->N, ctx->Np, ctx->R,
+                       ctx->Rp, ctx->gslices, rows_per_chunk);
 }
 
 int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
@@ -1466,7 +1474,9 @@ int init_ctx(pink_hip_ctx *ctx)
             // k is cut so that every CU gets about two waves; a block of four waves takes one slice
             uint32_t cuts = std::max(1u, (2u * (uint32_t)ctx->num_cu + tiles - 1) / tiles);
             cuts = std::min(cuts, std::max(1u, ctx->gKS / 4));
-            const uint32_t slices = (cuts + 3) / 4;
+            uint32_t slices = (cuts + 3) / 4;
+            // few k-steps per wave either way: one block per tile, which then finishes the tile itself
+            if ((ctx->gKS + 3) / 4 <= 8) slices = 1;
             ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
             ctx->gslices = (ctx->gKS + 4 * ctx->gks_per - 1) / (4 * ctx->gks_per);
         }
