@@ -799,35 +799,53 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
     long long sq = 0;
     const size_t plane_bytes = (size_t)(up.Np / 32) * up.KS * 64 * 16;
-    for (uint32_t j = j0 + tid; j < j1; j += 256) {
-        const float wv = w[j];
-        const float nv = __fsub_rn(wv, __fmul_rn(__fsub_rn(wv, x[j]), f));
-        w[j] = nv;
-        // keep the distance kernel's packed copy of the region current (inv = position of element
-        // j in the region, or none)
-        if (inv) {
-            const uint32_t k = inv[j];
-            if (k != 0xffffffffu) {
-                if (up.Pa) {
-                    const int q = quantise(nv, qfactor);
-                    const size_t byte = ((((size_t)(n >> 5) * up.KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
-                    if (up.u16) {
-                        const int c = q - 32768;
-                        const int h = c >> 8, l = (c & 255) - 128;
-                        up.Pa[byte] = (signed char)h;
-                        up.Pa[plane_bytes + byte] = (signed char)l;
-                        const long long v = 256 * h + l;
-                        sq += v * v;
-                    } else {
-                        const int h = q - 128;
-                        up.Pa[byte] = (signed char)h;
-                        sq += h * h;
-                    }
-                } else if (qfactor > 0.0f) {
-                    ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
-                } else {
-                    ((float *)somP)[(size_t)n * Epad + k] = nv;
-                }
+    // keep the distance kernel's packed copy of the region current (inv = position of element j in
+    // the region, or none)
+    auto refresh = [&](uint32_t k, float nv) {
+        if (k == 0xffffffffu) return;
+        if (up.Pa) {
+            const int q = quantise(nv, qfactor);
+            const size_t byte = ((((size_t)(n >> 5) * up.KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
+            if (up.u16) {
+                const int c = q - 32768;
+                const int h = c >> 8, l = (c & 255) - 128;
+                up.Pa[byte] = (signed char)h;
+                up.Pa[plane_bytes + byte] = (signed char)l;
+                const long long v = 256 * h + l;
+                sq += v * v;
+            } else {
+                const int h = q - 128;
+                up.Pa[byte] = (signed char)h;
+                sq += h * h;
+            }
+        } else if (qfactor > 0.0f) {
+            ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
+        } else {
+            ((float *)somP)[(size_t)n * Epad + k] = nv;
+        }
+    };
+    // Four elements per thread and round: all their loads are issued before the first store, so a
+    // thread keeps several cache lines in flight (the kernel lives on memory latency and bandwidth).
+    constexpr uint32_t U = 4;
+    for (uint32_t jb = j0 + tid; jb < j1; jb += 256 * U) {
+        float wv[U], xv[U];
+        uint32_t kk[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t j = jb + 256 * u;
+            if (j < j1) {
+                wv[u] = w[j];
+                xv[u] = x[j];
+                kk[u] = inv ? inv[j] : 0xffffffffu;
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t j = jb + 256 * u;
+            if (j < j1) {
+                const float nv = __fsub_rn(wv[u], __fmul_rn(__fsub_rn(wv[u], xv[u]), f));
+                w[j] = nv;
+                refresh(kk[u], nv);
             }
         }
     }
