@@ -326,6 +326,63 @@ def test_map_full_size_properties():
     assert np.array_equal(bits(heat3), bits(heat[:50]))
 
 
+def test_empty_inputs_are_no_ops():
+    w = synthetic.WORKLOADS["cfg4"]
+    som = synthetic.initial_som(w)
+    none = np.empty((0, w.channels, w.image_dim, w.image_dim), np.float32)
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(som)
+        assert ctx.train(none).shape == (0,)
+        assert np.array_equal(bits(ctx.get_som()), bits(som))
+    with capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                      w.ed_shape, w.ed_type) as ctx:
+        ctx.set_som(som)
+        heat, best = ctx.map(none)
+        assert heat.shape == (0, w.som_size) and best.shape == (0, w.som_size)
+
+
+@pytest.mark.parametrize("ed_type", [capi.UINT8, capi.UINT16])
+def test_out_of_range_pixels_saturate_like_the_oracle(ed_type):
+    """Values outside [0, 1] (undefined in the reference) quantise to the ends of the range on every
+    integer path, 1.0 exactly to the top value."""
+    N, C_, I, D, nrot, flip, ed = 20, 1, 24, 18, 40, True, 16
+    rng = np.random.default_rng(5)
+    som = (rng.random((N, D * D), dtype=np.float32) * 2 - 0.5).astype(np.float32)
+    imgs = (rng.random((6, C_, I, I), dtype=np.float32) * 2 - 0.5).astype(np.float32)
+    imgs[0, 0, :4, :4] = 1.0
+    som[0, :9] = [1.0, 0.0, -0.0, 2.0, -3.0, 1.0000001, 0.99999994, 0.5, 1e-9]
+    s = O.shape(N, C_, I, D, nrot, flip, ed, O.QUADRATIC, ed_type)
+    oheat, obest = O.map_images(s, som, imgs)
+    for choice in (capi.KERNEL_AUTO, capi.KERNEL_VALU, capi.KERNEL_MFMA_GEMM):
+        with capi.Context(N, C_, I, D, nrot, flip, ed, capi.QUADRATIC, ed_type, kernel_choice=choice) as ctx:
+            ctx.set_som(som)
+            heat, best = ctx.map(imgs)
+        assert np.array_equal(bits(heat), bits(oheat)) and np.array_equal(best, obest), choice
+
+
+def test_train_full_size_is_deterministic_and_counts_every_image():
+    """cfg 4 at its full size (60 000 images), where the oracle is not run: two runs agree bit for
+    bit, every image gets a best-matching neuron, and a second epoch moves the map less than the first."""
+    w = synthetic.WORKLOADS["cfg4"]
+    imgs = synthetic.images(w)
+    som0 = synthetic.initial_som(w)
+    runs = []
+    for _ in range(2):
+        with synthetic.make_context(w) as ctx:
+            ctx.set_som(som0)
+            bmu = ctx.train(imgs)
+            som1 = ctx.get_som()
+            ctx.train(imgs)
+            som2 = ctx.get_som()
+        runs.append((bmu, som1, som2))
+    assert np.array_equal(runs[0][0], runs[1][0]) and np.array_equal(bits(runs[0][1]), bits(runs[1][1]))
+    bmu, som1, som2 = runs[0]
+    assert bmu.shape == (w.n_images,) and bmu.max() < w.som_size
+    assert np.bincount(bmu, minlength=w.som_size).sum() == w.n_images
+    assert np.isfinite(som2).all()
+    assert np.abs(som2 - som1).mean() < np.abs(som1 - som0).mean()
+
+
 def test_mfma_kernel_refused_where_it_does_not_apply():
     with pytest.raises(capi.PinkError):
         capi.Context(200, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.UINT8, kernel_choice=capi.KERNEL_MFMA)
