@@ -166,6 +166,9 @@ int pink_hip_device_info(char *buf, size_t len);
  * functors of UtilitiesLib/DistributionFunctor.cpp:19-59 (`sigma` is the step width
  * for PINK_HIP_STEP).  factors_out holds N*N floats, N = pink_hip_som_size(...). */
 uint32_t pink_hip_som_size(uint32_t layout, const uint32_t *dims, uint32_t ndims);
+/* SOMLayout::get_distance(i, j) for all pairs (N*N floats): what a caller with its own
+ * distribution function (the std::function<float(float)> of Trainer.h:211) evaluates it on. */
+int pink_hip_layout_distances(uint32_t layout, const uint32_t *dims, uint32_t ndims, float *distances_out);
 int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t ndims, uint32_t functor,
                                  float sigma, float damping, float max_update_distance, float *factors_out);
 

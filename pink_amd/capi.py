@@ -28,7 +28,7 @@ EXPORTS = (
     "pink_hip_map", "pink_hip_map_device", "pink_hip_synchronize", "pink_hip_rotate",
     "pink_hip_distance", "pink_hip_region_size", "pink_hip_distance_kernel", "pink_hip_set_profiling",
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
-    "pink_hip_make_update_factors",
+    "pink_hip_make_update_factors", "pink_hip_layout_distances",
 )
 
 
@@ -84,6 +84,7 @@ def lib():
         L.pink_hip_som_size.argtypes = [u32, u32p, u32]
         L.pink_hip_som_size.restype = u32
         L.pink_hip_make_update_factors.argtypes = [u32, u32p, u32, u32, C.c_float, C.c_float, C.c_float, f32p]
+        L.pink_hip_layout_distances.argtypes = [u32, u32p, u32, f32p]
         _lib = L
     return _lib
 
@@ -120,6 +121,19 @@ def make_update_factors(layout, dims, functor, sigma, damping=0.0, max_update_di
                                             max_update_distance, _f32(out))
     if rc != 0:
         raise PinkError(rc, "pink_hip_make_update_factors: invalid argument")
+    return out
+
+
+def layout_distances(layout, dims):
+    """SOMLayout::get_distance for all neuron pairs, (N, N) float32."""
+    dims = np.ascontiguousarray(dims, np.uint32)
+    n = som_size(layout, dims)
+    if n == 0:
+        raise PinkError(-1, "invalid SOM layout dimensions")
+    out = np.empty((n, n), np.float32)
+    rc = lib().pink_hip_layout_distances(layout, _u32(dims), len(dims), _f32(out))
+    if rc != 0:
+        raise PinkError(rc, "pink_hip_layout_distances: invalid argument")
     return out
 
 

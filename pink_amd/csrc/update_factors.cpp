@@ -107,12 +107,8 @@ uint32_t pink_hip_som_size(uint32_t layout, const uint32_t *dims, uint32_t ndims
     return n;
 }
 
-int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t ndims, uint32_t functor,
-                                 float sigma, float damping, float max_update_distance, float *factors_out)
+static Grid make_grid(uint32_t layout, const uint32_t *dims, uint32_t ndims)
 {
-    const uint32_t N = pink_hip_som_size(layout, dims, ndims);
-    if (N == 0 || !factors_out || functor > PINK_HIP_MEXICAN_HAT) return PINK_HIP_EINVAL;
-    if (functor == PINK_HIP_MEXICAN_HAT && sigma <= 0.0f) return PINK_HIP_EINVAL;   // DistributionFunctor.cpp:50
     Grid g{};
     g.layout = layout;
     g.ndims = ndims;
@@ -125,6 +121,26 @@ int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t
             g.row_offset[r + 1] = g.row_offset[r] + dims[0] - away;
         }
     }
+    return g;
+}
+
+int pink_hip_layout_distances(uint32_t layout, const uint32_t *dims, uint32_t ndims, float *distances_out)
+{
+    const uint32_t N = pink_hip_som_size(layout, dims, ndims);
+    if (N == 0 || !distances_out) return PINK_HIP_EINVAL;
+    const Grid g = make_grid(layout, dims, ndims);
+    for (uint32_t i = 0; i < N; ++i)
+        for (uint32_t j = 0; j < N; ++j) distances_out[static_cast<size_t>(i) * N + j] = g.distance(i, j);
+    return PINK_HIP_OK;
+}
+
+int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t ndims, uint32_t functor,
+                                 float sigma, float damping, float max_update_distance, float *factors_out)
+{
+    const uint32_t N = pink_hip_som_size(layout, dims, ndims);
+    if (N == 0 || !factors_out || functor > PINK_HIP_MEXICAN_HAT) return PINK_HIP_EINVAL;
+    if (functor == PINK_HIP_MEXICAN_HAT && sigma <= 0.0f) return PINK_HIP_EINVAL;   // DistributionFunctor.cpp:50
+    const Grid g = make_grid(layout, dims, ndims);
     for (uint32_t i = 0; i < N; ++i)
         for (uint32_t j = 0; j < N; ++j) {
             const float d = g.distance(i, j);
