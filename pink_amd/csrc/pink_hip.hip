@@ -1211,23 +1211,29 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 #undef LAUNCH_TN
 }
 
+// Distances of B images starting at image slot `slot`.  One image (training): k is cut into
+// ctx->gslices slices so that the chip is filled.  Several images (mapping): the images fill the
+// chip, every block takes the whole k range of its tile and finishes it, one launch for all.
 template <bool U16>
-void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot)
+void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     const uint32_t planes = U16 ? 2 : 1;
     const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
     const uint32_t tiles_per_xcd = ((ctx->Rp / 64) * (ctx->Np / 64) + 7) / 8;
+    const uint32_t slices = B > 1 ? 1 : ctx->gslices;
+    const uint32_t ks_per = B > 1 ? (ctx->gKS + 3) / 4 : ctx->gks_per;
     GemmFinish fin{};
     long long *na = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, *na_other = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
     const long long *nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
-    if (ctx->gslices == 1) {
+    fin.nb = nb;
+    if (slices == 1) {
         // a block sees the whole k range: it finishes its tile itself
-        fin.key = key; fin.na = na; fin.na_other = na_other; fin.nb = nb; fin.N = ctx->N; fin.R = ctx->R;
+        fin.key = key; fin.na = na; fin.na_other = na_other; fin.N = ctx->N; fin.R = ctx->R;
     }
-    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * ctx->gslices), dim3(256), 0, ctx->stream, ctx->d_gPa, pb,
-                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ctx->gks_per, ctx->gslices, tiles_per_xcd, fin);
-    if (ctx->gslices == 1) return;
+    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, ctx->d_gPa, pb,
+                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, slices, tiles_per_xcd, fin);
+    if (slices == 1) return;
     const uint32_t rows_per_chunk = 32;
     hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
                        dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, na, na_other, nb, key, ctx->N, ctx->Np, ctx->R,
@@ -1238,10 +1244,8 @@ int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     Timed t(ctx, kClsDist);
     if (ctx->gemm) {
-        for (uint32_t b = 0; b < B; ++b) {
-            if (ctx->cfg.ed_type == PINK_HIP_UINT16) launch_dist_gemm<true>(ctx, slot + b);
-            else launch_dist_gemm<false>(ctx, slot + b);
-        }
+        if (ctx->cfg.ed_type == PINK_HIP_UINT16) launch_dist_gemm<true>(ctx, slot, B);
+        else launch_dist_gemm<false>(ctx, slot, B);
         return launch_check(ctx, "k_dist_gemm_int");
     }
     // the vector-ALU kernels below read d_somP / d_rotT: never reached without them
