@@ -169,6 +169,15 @@ uint32_t pink_hip_som_size(uint32_t layout, const uint32_t *dims, uint32_t ndims
 /* SOMLayout::get_distance(i, j) for all pairs (N*N floats): what a caller with its own
  * distribution function (the std::function<float(float)> of Trainer.h:211) evaluates it on. */
 int pink_hip_layout_distances(uint32_t layout, const uint32_t *dims, uint32_t ndims, float *distances_out);
+
+/* Host-only helpers for the callers either side of the path.
+ * pink_hip_shuffled_order: the order in which DataIteratorShuffled visits a data file of n entries
+ * (DataIteratorShuffled.h:62-69: iota, std::default_random_engine(seed), std::mt19937 seeded with its
+ * first draw, std::shuffle); the training loop uses seed + iteration (Pink/main_generic.h:83-84).
+ * pink_hip_fill_random_uniform: fill_random_uniform of UtilitiesLib/Filler.h:16-25, the SOM
+ * initialisation "random" (SOM.h:79-80): std::mt19937(seed), uniform_real_distribution<float>(0, 1). */
+int pink_hip_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order_out);
+int pink_hip_fill_random_uniform(float *values_out, size_t length, uint32_t seed);
 int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t ndims, uint32_t functor,
                                  float sigma, float damping, float max_update_distance, float *factors_out);
 

@@ -238,6 +238,18 @@ def fill_random_uniform(n, seed):
     return a
 
 
+def shuffled_order(seed, n):
+    a = np.empty(n, np.uint32)
+    lib().pink_oracle_shuffled_order(C.c_uint64(seed), C.c_uint32(n), _p(a, C.c_uint32))
+    return a
+
+
+def ref_shuffled_order(seed, n, shuffle=True):
+    a = np.empty(n, np.uint32)
+    ref().ref_shuffled_order(C.c_uint64(seed), C.c_uint32(n), C.c_int(int(shuffle)), _p(a, C.c_uint32))
+    return a
+
+
 def mt19937_raw(seed, n):
     a = np.empty(n, np.uint32)
     lib().pink_oracle_mt19937_raw(C.c_uint32(seed), _p(a, C.c_uint32), C.c_size_t(n))

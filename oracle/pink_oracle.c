@@ -593,6 +593,61 @@ void pink_oracle_fill_random_uniform(float *a, size_t length, uint32_t seed)
     }
 }
 
+/* A draw of std::uniform_int_distribution<size_t>(0, range - 1) from a 32-bit generator as
+ * libstdc++ 11 makes it (bits/uniform_int_dist.h, the multiply-and-reject method taken when the
+ * generator's range is exactly 2^32): high word of word * range, redrawn while the low word falls
+ * under 2^32 mod range.  `range` below 2^32. */
+static uint32_t uniform_below(mt19937_t *g, uint64_t range)
+{
+    uint64_t product = (uint64_t)mt_next(g) * range;
+    uint32_t low = (uint32_t)product;
+    if (low < range) {
+        const uint32_t threshold = (uint32_t)(-(uint32_t)range) % (uint32_t)range;
+        while (low < threshold) {
+            product = (uint64_t)mt_next(g) * range;
+            low = (uint32_t)product;
+        }
+    }
+    return (uint32_t)(product >> 32);
+}
+
+static void swap_u32(uint32_t *a, uint32_t *b) { const uint32_t t = *a; *a = *b; *b = t; }
+
+/* SelfOrganizingMapLib/DataIteratorShuffled.h:62-69 : iota, std::default_random_engine(seed)
+ * (minstd_rand0: x = seed mod (2^31 - 1), 1 if that is 0; next x = 16807 x mod (2^31 - 1)), a
+ * std::mt19937 seeded with its first draw, std::shuffle.  std::shuffle as libstdc++ 11 has it
+ * (bits/stl_algo.h): while the square of the length fits the generator's range, two swap positions
+ * come out of one draw (position i with one of [0, i], position i + 1 with one of [0, i + 1]; an even
+ * length first swaps position 1 alone); otherwise one draw per position.  The order is a property of
+ * that library version, as it is for the reference. */
+void pink_oracle_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order)
+{
+    for (uint32_t i = 0; i < n; ++i) order[i] = i;
+    if (n == 0) return;
+    uint64_t x = seed % 2147483647u;
+    if (x == 0) x = 1;
+    x = (16807u * x) % 2147483647u;
+    mt19937_t g;
+    mt_seed(&g, (uint32_t)x);
+    const uint64_t generator_range = 4294967295u;
+    if (generator_range / n >= n) {
+        uint32_t i = 1;
+        if (n % 2 == 0) {
+            swap_u32(&order[i], &order[uniform_below(&g, 2)]);
+            ++i;
+        }
+        while (i < n) {
+            const uint64_t first_range = (uint64_t)i + 1, second_range = first_range + 1;
+            const uint32_t both = uniform_below(&g, first_range * second_range);
+            swap_u32(&order[i], &order[both / second_range]);
+            swap_u32(&order[i + 1], &order[both % second_range]);
+            i += 2;
+        }
+        return;
+    }
+    for (uint32_t i = 1; i < n; ++i) swap_u32(&order[i], &order[uniform_below(&g, (uint64_t)i + 1)]);
+}
+
 /* Threads the OpenMP loops above will use (1 without OpenMP). */
 int pink_oracle_num_threads(void)
 {

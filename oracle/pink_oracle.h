@@ -121,6 +121,8 @@ int pink_oracle_map(const pink_oracle_shape *s, const float *som, const float *i
 /* ---- random filler -------------------------------------------------------- */
 void pink_oracle_fill_random_uniform(float *a, size_t length, uint32_t seed);
 void pink_oracle_mt19937_raw(uint32_t seed, uint32_t *out, size_t n);
+/* Visiting order of the shuffled data iterator for `n` entries. */
+void pink_oracle_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order);
 
 int pink_oracle_num_threads(void);
 

@@ -24,6 +24,8 @@
 #include "ImageProcessingLib/circular_euclidean_distance.h"
 #include "UtilitiesLib/DistributionFunctor.h"
 #include "UtilitiesLib/Filler.h"
+#include "SelfOrganizingMapLib/DataIteratorShuffled.h"
+#include <sstream>
 
 using namespace pink;
 
@@ -153,5 +155,21 @@ float ref_functor(uint32_t kind, float sigma, float damping, float distance)
 }
 
 void ref_fill_random_uniform(float* a, size_t n, uint32_t seed) { fill_random_uniform(a, n, seed); }
+
+/// The visiting order of the reference's DataIteratorShuffled over an in-memory data file of
+/// n one-pixel images whose pixel is the entry's index.
+void ref_shuffled_order(uint64_t seed, uint32_t n, int shuffle, uint32_t* order)
+{
+    std::stringstream ss;
+    const int head[8] = {2, 0, 0, static_cast<int>(n), 0, 2, 1, 1};
+    ss.write(reinterpret_cast<const char*>(head), sizeof(head));
+    for (uint32_t i = 0; i < n; ++i) {
+        const float v = static_cast<float>(i);
+        ss.write(reinterpret_cast<const char*>(&v), sizeof(v));
+    }
+    DataIteratorShuffled<CartesianLayout<2>, float> it(ss, seed, shuffle != 0);
+    const DataIteratorShuffled<CartesianLayout<2>, float> end(ss, true);
+    for (uint32_t i = 0; it != end && i < n; ++it, ++i) order[i] = static_cast<uint32_t>((*it)[0]);
+}
 
 } // extern "C"

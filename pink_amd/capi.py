@@ -28,7 +28,8 @@ EXPORTS = (
     "pink_hip_map", "pink_hip_map_device", "pink_hip_synchronize", "pink_hip_rotate",
     "pink_hip_distance", "pink_hip_region_size", "pink_hip_distance_kernel", "pink_hip_set_profiling",
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
-    "pink_hip_make_update_factors", "pink_hip_layout_distances",
+    "pink_hip_make_update_factors", "pink_hip_layout_distances", "pink_hip_shuffled_order",
+    "pink_hip_fill_random_uniform",
 )
 
 
@@ -85,6 +86,8 @@ def lib():
         L.pink_hip_som_size.restype = u32
         L.pink_hip_make_update_factors.argtypes = [u32, u32p, u32, u32, C.c_float, C.c_float, C.c_float, f32p]
         L.pink_hip_layout_distances.argtypes = [u32, u32p, u32, f32p]
+        L.pink_hip_shuffled_order.argtypes = [C.c_uint64, u32, u32p]
+        L.pink_hip_fill_random_uniform.argtypes = [f32p, C.c_size_t, u32]
         _lib = L
     return _lib
 
@@ -134,6 +137,24 @@ def layout_distances(layout, dims):
     rc = lib().pink_hip_layout_distances(layout, _u32(dims), len(dims), _f32(out))
     if rc != 0:
         raise PinkError(rc, "pink_hip_layout_distances: invalid argument")
+    return out
+
+
+def shuffled_order(seed, n):
+    """The order in which the reference's shuffled iterator visits n entries (DataIteratorShuffled.h:62-69)."""
+    out = np.empty(n, np.uint32)
+    rc = lib().pink_hip_shuffled_order(int(seed), n, _u32(out))
+    if rc != 0:
+        raise PinkError(rc, "pink_hip_shuffled_order: invalid argument")
+    return out
+
+
+def fill_random_uniform(length, seed):
+    """fill_random_uniform (UtilitiesLib/Filler.h:16-25): `length` float32 in [0, 1) from std::mt19937(seed)."""
+    out = np.empty(length, np.float32)
+    rc = lib().pink_hip_fill_random_uniform(_f32(out), length, int(seed))
+    if rc != 0:
+        raise PinkError(rc, "pink_hip_fill_random_uniform: invalid argument")
     return out
 
 

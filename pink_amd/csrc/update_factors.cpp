@@ -6,9 +6,12 @@
 // (CartesianLayout.h:47-60,103-129; HexagonalLayout.h:79-104) and one of the functors of
 // src/UtilitiesLib/DistributionFunctor.cpp:19-59.  All arithmetic is float, with the same
 // libm calls, so the matrix equals the reference's bit for bit on the same libm.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdlib>
+#include <numeric>
+#include <random>
 #include <vector>
 
 #include "pink_hip.h"
@@ -148,6 +151,27 @@ int pink_hip_make_update_factors(uint32_t layout, const uint32_t *dims, uint32_t
             if (max_update_distance <= 0 || d < max_update_distance) f = neighbourhood(functor, sigma, damping, d);
             factors_out[static_cast<size_t>(i) * N + j] = f;
         }
+    return PINK_HIP_OK;
+}
+
+int pink_hip_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order_out)
+{
+    if (n && !order_out) return PINK_HIP_EINVAL;
+    // The order is whatever the C++ library's engines and std::shuffle give for these calls
+    // (DataIteratorShuffled.h:62-69): the library decides, as it does for the reference.
+    std::iota(order_out, order_out + n, 0u);
+    std::default_random_engine engine(seed);
+    std::mt19937 generator(engine());
+    std::shuffle(order_out, order_out + n, generator);
+    return PINK_HIP_OK;
+}
+
+int pink_hip_fill_random_uniform(float *values_out, size_t length, uint32_t seed)
+{
+    if (length && !values_out) return PINK_HIP_EINVAL;
+    std::mt19937 generator(seed);
+    std::uniform_real_distribution<float> uniform(0.0f);
+    for (size_t i = 0; i < length; ++i) values_out[i] = uniform(generator);
     return PINK_HIP_OK;
 }
 

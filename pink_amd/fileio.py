@@ -187,14 +187,53 @@ def read_rot_flip_file(path):
     return som_dims, rec["flip"].copy(), rec["angle"].copy()
 
 
-def train_file(trainer, data_path, som, result_path, number_of_iterations=1, header=b""):
-    """The training loop of Pink --train with --input-shuffle-off (main_generic.h:80-116): every
-    image of the data file in file order, `number_of_iterations` times, then the SOM file.
-    `trainer` and `som` are pink_amd.pink objects."""
+def initial_som(som_layout, som_dims, neuron_dims, init="zero", seed=1234, som_file=None):
+    """The SOM the reference starts training from (SOM.h:69-98), as (number_of_neurons, prod(neuron_dims))
+    float32: "zero"; "random" = fill_random_uniform(seed); "random_with_preferred_direction" = the same with
+    the diagonal of the first neuron_dims[-1] x neuron_dims[-1] block of every neuron set to 1; "file" = the
+    weights of `som_file`, found as the reference finds them: behind the text header and 9 +
+    <SOM dimensionality> integers (SOM.h:94, which assumes two neuron dimensions)."""
+    from . import capi
+    layout = capi.HEXAGONAL if som_layout == "hexagonal-2d" else capi.CARTESIAN
+    n = capi.som_size(layout, np.asarray(list(som_dims), np.uint32))
+    if n == 0:
+        raise FormatError("invalid SOM dimensions")
+    per_neuron = int(np.prod(neuron_dims))
+    if init == "zero":
+        return np.zeros((n, per_neuron), np.float32)
+    if init in ("random", "random_with_preferred_direction"):
+        som = capi.fill_random_uniform(n * per_neuron, seed).reshape(n, per_neuron)
+        if init == "random_with_preferred_direction":
+            d = int(neuron_dims[-1])
+            som[:, np.arange(d) * d + np.arange(d)] = 1.0
+        return som
+    if init == "file":
+        with open(som_file, "rb") as f:
+            read_header(f)
+            f.seek(4 * (9 + len(_som_dims(som_layout, list(som_dims)))), 1)
+            data = np.frombuffer(f.read(4 * n * per_neuron), np.float32)
+        if data.size != n * per_neuron:
+            raise FormatError("SOM file is shorter than the SOM")
+        return data.reshape(n, per_neuron).copy()
+    raise FormatError("unknown SOM initialisation " + repr(init))
+
+
+def train_file(trainer, data_path, som, result_path, number_of_iterations=1, header=b"", shuffle=True, seed=1234):
+    """The training loop of Pink --train (main_generic.h:79-110): `number_of_iterations` passes over the
+    data file, pass i in the order of DataIteratorShuffled(seed + i) -- or in file order with
+    shuffle=False (--input-shuffle-off) -- then the SOM file.  `trainer` and `som` are pink_amd.pink
+    objects."""
+    from . import capi
     data = DataFile(data_path)
     layout = "cartesian-3d" if len(data.dimensions) == 3 else "cartesian-2d"
-    for _ in range(number_of_iterations):
-        trainer.train(data.images, layout)
+    step = max(1, (1 << 28) // max(1, 4 * int(np.prod(data.dimensions))))      # images gathered per call
+    for i in range(number_of_iterations):
+        if not shuffle:
+            trainer.train(data.images, layout)
+            continue
+        order = capi.shuffled_order(seed + i, len(data))
+        for begin in range(0, len(order), step):
+            trainer.train(data.images[order[begin:begin + step]], layout)
     trainer.update_som()
     write_som_file(result_path, np.asarray(som), som.som_layout, som._dims, som.neuron_shape, header)
     return trainer.get_update_info()

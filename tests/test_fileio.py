@@ -3,8 +3,11 @@
 The expected bytes are written out field by field from the reference's own writers and test
 fixtures (cited per test), not produced by the module under test.
 """
+import json
 import math
+import os
 import struct
+import zlib
 
 import numpy as np
 import pytest
@@ -115,6 +118,51 @@ def test_mapping_and_rot_flip_files(tmp_path):
     assert flips.tolist() == [[0, 0, 0, 1], [1, 1, 0, 1]] and angles.shape == (2, 4)
 
 
+def _shuffle_vectors():
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "shuffle_orders.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("make", [capi.shuffled_order, O.shuffled_order], ids=["library", "oracle"])
+def test_shuffled_order_against_the_reference_vectors(make):
+    # tests/golden/shuffle_orders.json holds orders taken from the reference's own iterator
+    for v in _shuffle_vectors():
+        order = make(v["seed"], v["n"])
+        assert sorted(order.tolist()) == list(range(v["n"]))
+        assert order[:len(v.get("order", v.get("head")))].tolist() == v.get("order", v.get("head")), v
+        assert zlib.crc32(order.astype("<u4").tobytes()) == v["crc32"], v
+    # test/SelfOrganizingMapTest/DataIteratorShuffled.cpp:19-35: seed 2 leaves two entries in file order
+    assert make(2, 2).tolist() == [0, 1]
+    assert make(7, 0).size == 0
+    # the training loop reseeds with seed + iteration (main_generic.h:83-84): the passes differ
+    assert not np.array_equal(make(1234, 50), make(1235, 50))
+
+
+def test_initial_som_kinds(tmp_path):
+    # SOM.h:77-96
+    z = fileio.initial_som("cartesian-2d", (3, 2), (4, 4), "zero")
+    assert z.shape == (6, 16) and not z.any()
+    r = fileio.initial_som("hexagonal-2d", (5,), (2, 4, 4), "random", seed=77)
+    assert r.shape == (19, 32)
+    assert np.array_equal(r.ravel(), O.fill_random_uniform(19 * 32, 77))
+    # Filler probe of the reference with seed 1234
+    assert np.allclose(fileio.initial_som("cartesian-2d", (1, 1), (2, 2), "random")[0],
+                       [0.191519, 0.497664, 0.622109, 0.817838], atol=1e-6)
+    d = fileio.initial_som("cartesian-2d", (2, 2), (3, 3), "random_with_preferred_direction", seed=5)
+    plain = O.fill_random_uniform(4 * 9, 5).reshape(4, 9)
+    assert np.array_equal(d[:, [0, 4, 8]], np.ones((4, 3), np.float32))
+    assert np.array_equal(np.delete(d, [0, 4, 8], axis=1), np.delete(plain, [0, 4, 8], axis=1))
+    # "file": weights behind the header and 9 + <SOM dimensionality> integers
+    w = np.arange(4 * 9, dtype=np.float32).reshape(4, 9)
+    fileio.write_som_file(tmp_path / "init.bin", w, "cartesian-2d", (2, 2), (3, 3), b"# x\n# END OF HEADER\n")
+    assert np.array_equal(fileio.initial_som("cartesian-2d", (2, 2), (3, 3), "file", som_file=tmp_path / "init.bin"), w)
+    (tmp_path / "short.bin").write_bytes(b"")
+    with pytest.raises(fileio.FormatError):
+        fileio.initial_som("cartesian-2d", (2, 2), (3, 3), "file", som_file=tmp_path / "short.bin")
+    with pytest.raises(fileio.FormatError):
+        fileio.initial_som("cartesian-2d", (2, 2), (3, 3), "spiral")
+
+
 @pytest.mark.gpu
 def test_train_and_map_from_files_against_the_oracle(tmp_path):
     rng = np.random.default_rng(21)
@@ -124,12 +172,23 @@ def test_train_and_map_from_files_against_the_oracle(tmp_path):
     som = pink.SOM(np_som.copy(), som_layout="hexagonal-2d")
     trainer = pink.Trainer(som, pink.GaussianFunctor(1.1, 0.2), number_of_rotations=16, euclidean_distance_dim=10,
                            euclidean_distance_shape=pink.CIRCULAR, euclidean_distance_type=pink.UINT16)
-    counts = fileio.train_file(trainer, tmp_path / "data.bin", som, tmp_path / "som.bin", number_of_iterations=2)
+    counts = fileio.train_file(trainer, tmp_path / "data.bin", som, tmp_path / "som.bin", number_of_iterations=2,
+                               shuffle=False)
     # the same two epochs with the oracle
     F = capi.make_update_factors(capi.HEXAGONAL, [5], capi.GAUSSIAN, 1.1, 0.2)
     s = O.shape(19, 1, 20, 14, 16, True, 10, O.CIRCULAR, capi.UINT16)
     want = np_som.reshape(19, -1).copy()
     bmu = np.concatenate([O.train(s, want, images[:, None], F), O.train(s, want, images[:, None], F)])
+    # and two shuffled epochs (the default, seed 1234): pass i in the oracle's order for seed + i
+    som_s = pink.SOM(np_som.copy(), som_layout="hexagonal-2d")
+    trainer_s = pink.Trainer(som_s, pink.GaussianFunctor(1.1, 0.2), number_of_rotations=16, euclidean_distance_dim=10,
+                             euclidean_distance_shape=pink.CIRCULAR, euclidean_distance_type=pink.UINT16)
+    counts_s = fileio.train_file(trainer_s, tmp_path / "data.bin", som_s, tmp_path / "som_shuffled.bin", 2)
+    want_s = np_som.reshape(19, -1).copy()
+    bmu_s = np.concatenate([O.train(s, want_s, images[O.shuffled_order(1234 + i, 12)][:, None], F) for i in range(2)])
+    assert np.array_equal(counts_s, np.bincount(bmu_s, minlength=19))
+    assert np.array_equal(fileio.read_som_file(tmp_path / "som_shuffled.bin")[3].view(np.uint32), want_s.view(np.uint32))
+    assert not np.array_equal(want_s, want)
     assert np.array_equal(counts, np.bincount(bmu, minlength=19))
     header, som_dims, neuron_dims, got = fileio.read_som_file(tmp_path / "som.bin")
     assert som_dims == [5, 5] and neuron_dims == [14, 14]

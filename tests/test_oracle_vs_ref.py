@@ -127,3 +127,14 @@ def test_filler_bit_exact(ref_mod):
         want = np.empty(n, np.float32)
         O.ref().ref_fill_random_uniform(want.ctypes.data_as(C.POINTER(C.c_float)), C.c_size_t(n), C.c_uint32(seed))
         assert np.array_equal(O.fill_random_uniform(n, seed).view(np.uint32), want.view(np.uint32))
+
+
+def test_shuffled_order_matches_the_reference_iterator(ref_mod):
+    O = ref_mod
+    # both branches of std::shuffle (two positions per draw up to 65536 entries, one beyond), odd and even
+    # lengths, a seed beyond 32 bits, the seeds 0 and 2^31 - 1 that the first engine maps to 1
+    for seed, n in ((2, 2), (1234, 10), (1234, 2001), (0, 7), (2147483647, 100), (2 ** 40 + 3, 1000),
+                    (99, 65536), (99, 65537), (5, 70001), (7, 1), (3, 3)):
+        assert np.array_equal(O.shuffled_order(seed, n), O.ref_shuffled_order(seed, n)), (seed, n)
+    assert O.ref_shuffled_order(5, 6, False).tolist() == [0, 1, 2, 3, 4, 5]
+
