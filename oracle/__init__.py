@@ -250,6 +250,12 @@ def ref_shuffled_order(seed, n, shuffle=True):
     return a
 
 
+def ref_progress_ticks(total, max_prints):
+    a = np.empty(total, np.int32)
+    k = ref().ref_progress_ticks(C.c_int(total), C.c_int(max_prints), _p(a, C.c_int32))
+    return a[:k].tolist()
+
+
 def mt19937_raw(seed, n):
     a = np.empty(n, np.uint32)
     lib().pink_oracle_mt19937_raw(C.c_uint32(seed), _p(a, C.c_uint32), C.c_size_t(n))

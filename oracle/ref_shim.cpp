@@ -25,6 +25,7 @@
 #include "UtilitiesLib/DistributionFunctor.h"
 #include "UtilitiesLib/Filler.h"
 #include "SelfOrganizingMapLib/DataIteratorShuffled.h"
+#include "UtilitiesLib/ProgressBar.h"
 #include <sstream>
 
 using namespace pink;
@@ -170,6 +171,18 @@ void ref_shuffled_order(uint64_t seed, uint32_t n, int shuffle, uint32_t* order)
     DataIteratorShuffled<CartesianLayout<2>, float> it(ss, seed, shuffle != 0);
     const DataIteratorShuffled<CartesianLayout<2>, float> end(ss, true);
     for (uint32_t i = 0; it != end && i < n; ++it, ++i) order[i] = static_cast<uint32_t>((*it)[0]);
+}
+
+/// The ticks at which the training loop of Pink/main_generic.h:78-90 finds ProgressBar::valid() true
+/// (checked after each image, before the increment); returns their number.
+int ref_progress_ticks(int total, int max_prints, int* ticks_out)
+{
+    std::stringstream sink;
+    ProgressBar bar(total, 70, max_prints, sink);
+    int k = 0;
+    for (int t = 0; t < total; ++t, ++bar)
+        if (bar.valid()) ticks_out[k++] = t;
+    return k;
 }
 
 } // extern "C"

@@ -218,22 +218,69 @@ def initial_som(som_layout, som_dims, neuron_dims, init="zero", seed=1234, som_f
     raise FormatError("unknown SOM initialisation " + repr(init))
 
 
-def train_file(trainer, data_path, som, result_path, number_of_iterations=1, header=b"", shuffle=True, seed=1234):
-    """The training loop of Pink --train (main_generic.h:79-110): `number_of_iterations` passes over the
+def progress_ticks(number_of_ticks, max_number_of_progress_prints=10, width=70):
+    """The ticks t (images trained before, counted over all passes) at which the training loop finds
+    ProgressBar::valid() true after training image t, i.e. where it writes an intermediate SOM
+    (main_generic.h:78,86-90 with UtilitiesLib/ProgressBar.h:21-52,72-75)."""
+    if number_of_ticks < 1:
+        raise ValueError("ProgressBar: number_of_iterations must be larger than 0")
+    if max_number_of_progress_prints < 1:
+        raise ValueError("ProgressBar: max number of progress prints must be larger than 0")
+    prints = min(number_of_ticks, max_number_of_progress_prints)
+    if width < prints:
+        raise ValueError("ProgressBar: width must be equal or larger than number of progress prints")
+    section = number_of_ticks // prints
+    next_valid = section + (1 if number_of_ticks % prints else 0)
+    out = []
+    for tick in range(number_of_ticks):          # `tick` increments have happened when image `tick` is trained
+        if tick == next_valid:
+            out.append(tick)
+            next_valid += section
+    return out
+
+
+def train_file(trainer, data_path, som, result_path, number_of_iterations=1, header=b"", shuffle=True, seed=1234,
+               intermediate_storage="off", max_number_of_progress_prints=10):
+    """The training loop of Pink --train (main_generic.h:75-110): `number_of_iterations` passes over the
     data file, pass i in the order of DataIteratorShuffled(seed + i) -- or in file order with
-    shuffle=False (--input-shuffle-off) -- then the SOM file.  `trainer` and `som` are pink_amd.pink
-    objects."""
+    shuffle=False (--input-shuffle-off) -- then the SOM file.  intermediate_storage "overwrite" or "keep"
+    also writes the SOM at the progress ticks of the reference, into the result file or into
+    <result>_<count>.<ext> (main_generic.h:88-104).  `trainer` and `som` are pink_amd.pink objects."""
     from . import capi
+    if intermediate_storage not in ("off", "overwrite", "keep"):
+        raise ValueError("unknown intermediate storage type " + repr(intermediate_storage))
     data = DataFile(data_path)
+    n = len(data)
     layout = "cartesian-3d" if len(data.dimensions) == 3 else "cartesian-2d"
     step = max(1, (1 << 28) // max(1, 4 * int(np.prod(data.dimensions))))      # images gathered per call
+    stops = progress_ticks(n * number_of_iterations, max_number_of_progress_prints) if intermediate_storage != "off" and n else []
+    result_path = str(result_path)
+    count = 0
+
+    def store_intermediate():
+        nonlocal count
+        name = result_path
+        if intermediate_storage == "keep":
+            dot = name.rfind(".")            # std::string::insert at find_last_of("."): npos throws in the reference
+            if dot < 0:
+                raise ValueError("result file name has no '.' to put the count in front of")
+            name = name[:dot] + "_%d" % count + name[dot:]
+            count += 1
+        trainer.update_som()
+        write_som_file(name, np.asarray(som), som.som_layout, som._dims, som.neuron_shape, header)
+
     for i in range(number_of_iterations):
-        if not shuffle:
-            trainer.train(data.images, layout)
-            continue
-        order = capi.shuffled_order(seed + i, len(data))
-        for begin in range(0, len(order), step):
-            trainer.train(data.images[order[begin:begin + step]], layout)
+        order = capi.shuffled_order(seed + i, n) if shuffle else None
+        # the pass is cut after every image that is followed by an intermediate SOM, and into calls of `step` images
+        cuts = sorted({t - i * n + 1 for t in stops if i * n <= t < (i + 1) * n} | {n})
+        begin = 0
+        for cut in cuts:
+            while begin < cut:
+                end = min(cut, begin + step)
+                trainer.train(data.images[begin:end] if order is None else data.images[order[begin:end]], layout)
+                begin = end
+            if cut - 1 + i * n in stops:
+                store_intermediate()
     trainer.update_som()
     write_som_file(result_path, np.asarray(som), som.som_layout, som._dims, som.neuron_shape, header)
     return trainer.get_update_info()

@@ -163,6 +163,50 @@ def test_initial_som_kinds(tmp_path):
         fileio.initial_som("cartesian-2d", (2, 2), (3, 3), "spiral")
 
 
+def test_progress_ticks_of_the_reference_progress_bar():
+    # test/UtilitiesTest/ProgressBarTest.cpp:15-26: 100 ticks, 10 prints: valid after 10 increments, not before
+    assert fileio.progress_ticks(100, 10) == list(range(10, 100, 10))
+    # ProgressBarTest.cpp:52-64: 3 ticks, 2 prints: prints after the second and third increment; the loop
+    # checks before the increment, so only tick 2 is seen
+    assert fileio.progress_ticks(3, 2) == [2]
+    # ProgressBarTest.cpp:39-50: a single tick prints once, after the loop's check
+    assert fileio.progress_ticks(1, 10) == []
+    # ProgressBarTest.cpp:28-37
+    for bad in ((0, 10, 70), (10, 0, 70), (100, 10, 9)):
+        with pytest.raises(ValueError):
+            fileio.progress_ticks(*bad)
+
+
+@pytest.mark.gpu
+def test_intermediate_storage_writes_the_som_at_the_progress_ticks(tmp_path):
+    rng = np.random.default_rng(5)
+    images = rng.random((7, 12, 12), dtype=np.float32)
+    np_som = rng.random((2, 2, 8, 8), dtype=np.float32)
+    fileio.write_data_file(tmp_path / "data.bin", images)
+    F = capi.make_update_factors(capi.CARTESIAN, [2, 2], capi.GAUSSIAN, 1.1, 0.2)
+    s = O.shape(4, 1, 12, 8, 8, True, 6, O.QUADRATIC, capi.FLOAT)
+    order = np.concatenate([O.shuffled_order(9 + i, 7) for i in range(2)])        # 14 ticks, 3 prints: after 5 and 9
+    ticks = fileio.progress_ticks(14, 3)
+    assert ticks == [5, 9, 13]
+    for kind in ("keep", "overwrite"):
+        som = pink.SOM(np_som.copy())
+        trainer = pink.Trainer(som, pink.GaussianFunctor(1.1, 0.2), number_of_rotations=8, euclidean_distance_dim=6,
+                               euclidean_distance_type=pink.FLOAT)
+        fileio.train_file(trainer, tmp_path / "data.bin", som, tmp_path / (kind + ".bin"), 2, seed=9,
+                          intermediate_storage=kind, max_number_of_progress_prints=3)
+        want = np_som.reshape(4, -1).copy()
+        done = 0
+        for k, t in enumerate(ticks):
+            O.train(s, want, images[order[done:t + 1]][:, None], F)
+            done = t + 1
+            if kind == "keep":
+                got = fileio.read_som_file(tmp_path / ("keep_%d.bin" % k))[3]
+                assert np.allclose(got, want, rtol=1e-4, atol=1e-6), (k, t)        # float32 weights: 1e-4 relative
+        O.train(s, want, images[order[done:]][:, None], F)
+        assert np.allclose(fileio.read_som_file(tmp_path / (kind + ".bin"))[3], want, rtol=1e-4, atol=1e-6)
+    assert not (tmp_path / "overwrite_0.bin").exists() and not (tmp_path / "keep_3.bin").exists()
+
+
 @pytest.mark.gpu
 def test_train_and_map_from_files_against_the_oracle(tmp_path):
     rng = np.random.default_rng(21)

@@ -138,3 +138,9 @@ def test_shuffled_order_matches_the_reference_iterator(ref_mod):
         assert np.array_equal(O.shuffled_order(seed, n), O.ref_shuffled_order(seed, n)), (seed, n)
     assert O.ref_shuffled_order(5, 6, False).tolist() == [0, 1, 2, 3, 4, 5]
 
+
+def test_intermediate_storage_ticks_match_the_reference_progress_bar(ref_mod):
+    from pink_amd import fileio
+    for total, prints in ((100, 10), (3, 2), (1, 10), (7, 3), (8, 3), (24, 10), (2000, 10), (2001, 7), (69, 70), (500, 70)):
+        assert fileio.progress_ticks(total, prints) == ref_mod.ref_progress_ticks(total, prints), (total, prints)
+
