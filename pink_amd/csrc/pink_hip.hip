@@ -765,25 +765,54 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
     const uint32_t tid = threadIdx.x;
+    const uint32_t n = blockIdx.y, part = blockIdx.x;
+    // What the block will read does not depend on the best-matching neuron, only whether it is
+    // needed does: the first round of loads is issued ahead of the search, which then runs while
+    // they are in flight (a neuron with factor 0 drops them).
+    constexpr uint32_t U = 4;
+    // (loads return in issue order: the keys go first, so the search below waits for them alone)
     unsigned long long bv = ~0ull;
     uint32_t bi = 0xffffffffu;
-    for (uint32_t n = tid; n < N; n += 256) {
-        const unsigned long long v = key[n] >> shift;
-        if (v < bv) { bv = v; bi = n; }        // ascending n per thread: first minimum kept
+    for (uint32_t m = tid; m < N; m += 256) {
+        const unsigned long long v = key[m] >> shift;
+        if (v < bv) { bv = v; bi = m; }        // ascending index per thread: first minimum kept
     }
-    s_val[tid] = bv;
-    s_idx[tid] = bi;
-    __syncthreads();
-    for (uint32_t s = 128; s > 0; s >>= 1) {
-        if (tid < s) {
-            const unsigned long long ov = s_val[tid + s];
-            const uint32_t oi = s_idx[tid + s];
-            if (ov < s_val[tid] || (ov == s_val[tid] && oi < s_idx[tid])) { s_val[tid] = ov; s_idx[tid] = oi; }
+    const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
+    const float *__restrict__ x = rot + (size_t)r * S;
+    float *__restrict__ w = som + (size_t)n * S;
+    const uint32_t chunk = (S + parts - 1) / parts;
+    const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
+    float wv[U], xv[U];
+    uint32_t kk[U];
+    auto load_round = [&](uint32_t jb) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t j = jb + 256 * u;
+            if (j < j1) {
+                wv[u] = w[j];
+                xv[u] = x[j];
+                kk[u] = inv ? inv[j] : 0xffffffffu;
+            }
         }
-        __syncthreads();
+    };
+    load_round(j0 + tid);
+    // first minimum of the block: within a wave by shuffles, then across the four waves
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const unsigned long long ov = __shfl_xor(bv, o, 64);
+        const uint32_t oi = __shfl_xor(bi, o, 64);
+        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
-    const uint32_t bmu = s_idx[0];
-    const uint32_t n = blockIdx.y, part = blockIdx.x;
+    if ((tid & 63) == 0) { s_val[tid >> 6] = bv; s_idx[tid >> 6] = bi; }
+    __syncthreads();
+    bv = s_val[0]; bi = s_idx[0];
+#pragma unroll
+    for (int g = 1; g < 4; ++g) {
+        const unsigned long long ov = s_val[g];
+        const uint32_t oi = s_idx[g];
+        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const uint32_t bmu = bi;
     if (n == 0 && part == 0 && tid == 0) *bmu_out = bmu;
 
     const float f = factors[(size_t)bmu * N + n];
@@ -792,11 +821,6 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         if (up.Pa && part == 0 && tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], (unsigned long long)up.na_cur[n]);
         return;
     }
-    const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
-    const float *__restrict__ x = rot + (size_t)r * S;
-    float *__restrict__ w = som + (size_t)n * S;
-    const uint32_t chunk = (S + parts - 1) / parts;
-    const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
     long long sq = 0;
     const size_t plane_bytes = (size_t)(up.Np / 32) * up.KS * 64 * 16;
     // keep the distance kernel's packed copy of the region current (inv = position of element j in
@@ -826,19 +850,8 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     };
     // Four elements per thread and round: all their loads are issued before the first store, so a
     // thread keeps several cache lines in flight (the kernel lives on memory latency and bandwidth).
-    constexpr uint32_t U = 4;
     for (uint32_t jb = j0 + tid; jb < j1; jb += 256 * U) {
-        float wv[U], xv[U];
-        uint32_t kk[U];
-#pragma unroll
-        for (uint32_t u = 0; u < U; ++u) {
-            const uint32_t j = jb + 256 * u;
-            if (j < j1) {
-                wv[u] = w[j];
-                xv[u] = x[j];
-                kk[u] = inv ? inv[j] : 0xffffffffu;
-            }
-        }
+        if (jb != j0 + tid) load_round(jb);
 #pragma unroll
         for (uint32_t u = 0; u < U; ++u) {
             const uint32_t j = jb + 256 * u;
@@ -853,7 +866,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         // (f depends on the block only, so every thread of the block is here)
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
-        __syncthreads();                                   // s_val was last read as s_idx[0]'s partner above
+        __syncthreads();                                   // s_val was last read by the search above
         if ((tid & 63) == 0) s_val[tid >> 6] = (unsigned long long)sq;
         __syncthreads();
         if (tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], s_val[0] + s_val[1] + s_val[2] + s_val[3]);
