@@ -41,7 +41,7 @@ MEASURED_FMA_NOPACK_TFLOPS = 72.5
 # HBM bytes per image from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/cfg1_map_u8_hbm_traffic.txt),
 # scaled by the same counters' readings for a 256 MiB device-to-device copy (FETCH x2.0, WRITE x1.0).
 MEASURED_TRAFFIC_PER_IMAGE = {
-    ("cfg1", 3, "rotate"): 57.8e3 + 138.1e3,     # image + part of the geometry table read; units written
+    ("cfg1", 3, "rotate"): 53.7e3 + 103.8e3,     # image + part of the geometry table read; units written
     ("cfg1", 3, "distance"): 108.1e3 + 0.8e3,    # units read once; keys written
 }
 
@@ -74,8 +74,9 @@ def algorithmic_per_image(w, E, path):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default: 30 for the mapping workload, whose step takes a few ms, 3 for training)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 10 mapping, 1 training)")
     ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -100,6 +101,11 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     w = synthetic.WORKLOADS[args.workload]
+    # a mapping step is a few milliseconds of GPU time: enough of them that the clocks have settled
+    if args.steps is None:
+        args.steps = 30 if w.mode == "map" else 3
+    if args.warmup is None:
+        args.warmup = 10 if w.mode == "map" else 1
     n_images = args.images or w.n_images
     kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA,
                      "mfma_sym": capi.KERNEL_MFMA_SYM, "mfma_gemm": capi.KERNEL_MFMA_GEMM}[args.kernel]
@@ -143,11 +149,10 @@ def main():
         step()
     ctx.synchronize()
 
-    # ---- timed region: exactly `steps` steps, HIP events around every kernel launch ----
+    # ---- timed region: exactly `steps` steps, nothing but the path's own launches on the stream ----
     if w.mode == "train":
         ctx.set_som(som0)
-    profile_in_timed = w.mode == "map"          # a few hundred launches: event cost is nil
-    ctx.set_profiling(profile_in_timed)
+    ctx.set_profiling(False)
     torch.cuda.synchronize()
     ctx.synchronize()
     t_start = time.perf_counter()
@@ -156,15 +161,20 @@ def main():
     ctx.synchronize()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_start
-    if profile_in_timed:
-        times = ctx.kernel_times()
+    # ---- per-kernel durations: HIP events around every launch, on the context's stream, in a pass of
+    # their own right after the timed one (the event records cost a mapper several per cent of its
+    # throughput and a trainer, with thousands of launches per second, much more)
+    ctx.set_profiling(True)
+    if w.mode == "map":
+        for _ in range(args.steps):
+            step()
         prof_images = n_images * args.steps
+        measured = "the %d timed steps repeated with per-launch HIP events" % args.steps
     else:
-        # training issues thousands of launches per second: per-kernel events go in their own pass
         prof_images = min(n_images, 256)
-        ctx.set_profiling(True)
         ctx.train_device(d_imgs.data_ptr(), prof_images, d_bmu.data_ptr())
-        times = ctx.kernel_times()
+        measured = "separate pass of %d images with per-launch HIP events" % prof_images
+    times = ctx.kernel_times()
     ctx.set_profiling(False)
 
     value = n_images * args.steps / elapsed
@@ -206,7 +216,7 @@ def main():
         "traffic": round(traffic * imgs_per_launch) if traffic else None,
         "algorithmic_bytes_per_launch": round(alg[dominant]["bytes"] * imgs_per_launch),
         "avg_launch_ms": round(avg_ms, 6), "launches": launches, "images_per_launch": imgs_per_launch,
-        "measured": "timed region" if profile_in_timed else "separate pass of %d images" % prof_images,
+        "measured": measured,
         "share_of_kernel_time": round(ms / total_ms, 4),
         "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
         "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries",

@@ -126,11 +126,11 @@ __global__ __launch_bounds__(256) void k_rot_table(const float *__restrict__ cos
             }
         }
     }
-    // piece-interleaved so that the 64 lanes of a wave, which hold 64 consecutive pieces of a
-    // rotation, read consecutive 16-byte entries: weights [i][j][piece], offsets [i][j / 4][piece][j % 4]
-    const uint32_t pieces = Kp / 16, piece = k / 16, j = k % 16;
-    tab_w[((size_t)i * 16 + j) * pieces + piece] = w;
-    tab_idx[(((size_t)i * 4 + j / 4) * pieces + piece) * 4 + j % 4] = idx;
+    // rotation-interleaved so that the lanes of a wave, which hold the same piece of 32 consecutive
+    // rotations, read consecutive 16-byte entries: weights [piece][j][i], offsets [piece][j / 4][i][j % 4]
+    const uint32_t piece = k / 16, j = k % 16;
+    tab_w[((size_t)piece * 16 + j) * rows + i] = w;
+    tab_idx[(((size_t)piece * 4 + j / 4) * rows + i) * 4 + j % 4] = idx;
 }
 
 // Byte `byte` of `word` = q = uint8(x * 255), truncated and saturated to [0, 255] (NaN -> 0):
@@ -221,9 +221,12 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
     }
     __syncthreads();
 
+    // The two halves of a wave take the two pieces of one k-step for the 32 rotations of the tile:
+    // a wave's 64 pieces are one whole fragment, written as 1 KiB of consecutive addresses.
     const uint32_t pieces = KS * 2;                       // 16-element pieces per row
+    const uint32_t rows = RTP * 32;
     for (uint32_t t = threadIdx.x; t < 32 * pieces; t += blockDim.x) {
-        const uint32_t g = t / pieces, piece = t % pieces;
+        const uint32_t g = t % 32, piece = t / 32;
         const uint32_t i = rt * 32 + g;                   // base rotation
         const uint32_t k0 = piece * 16;
         uint32_t word[G][4];
@@ -233,16 +236,15 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
             for (int w4 = 0; w4 < 4; ++w4) word[gi][w4] = 0;
         uint32_t live[4] = {0, 0, 0, 0};
         if (i < nrr_eff) {
-            // (uniform per wave: a wave covers the pieces of whole rotations)
-            const uint4 *ti = (const uint4 *)tab_idx + (size_t)i * 4 * pieces + piece;
-            const float4 *tw = tab_w + (size_t)i * 16 * pieces + piece;
+            const uint4 *ti = (const uint4 *)tab_idx + (size_t)piece * 4 * rows + i;
+            const float4 *tw = tab_w + (size_t)piece * 16 * rows + i;
 #pragma unroll
             for (int w4 = 0; w4 < 4; ++w4) {
-                const uint4 iv = ti[w4 * pieces];
+                const uint4 iv = ti[w4 * rows];
                 const uint32_t ii[4] = {iv.x, iv.y, iv.z, iv.w};
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const float4 wv = tw[(4 * w4 + u) * pieces];
+                    const float4 wv = tw[(4 * w4 + u) * rows];
                     const float *tap = s_img + ii[u];
                     live[w4] |= (k0 + 4 * w4 + u < Ku ? 0xffu : 0u) << (8 * u);
                     // (all G images, also past the end of the batch: what is computed from LDS nobody
