@@ -133,7 +133,7 @@ struct PackArgs {
 };
 
 template <int PACK>
-__global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
+__global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
@@ -187,50 +187,54 @@ __global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ images
                     }
                 }
         } else if constexpr (PACK >= 2) {
+            // One work item = one 16-byte piece of one of the block's (up to 8) rows; the items of all
+            // rows are dealt to the threads in one sequence, so the last round is the only partial one.
+            // Four elements at a time: quantise (clamp, truncate), bytes gathered with v_perm, q - 128 (or
+            // the two bytes of q - 32768 with the low one shifted by 128) = the bytes XOR 0x80, squares by
+            // dot4: |256 h + l|^2 = 65536 h.h + 512 h.l + l.l.
             constexpr bool U16 = PACK == 3;
             constexpr uint32_t planes = U16 ? 2 : 1;
             const float factor = U16 ? 65535.0f : 255.0f;
             const size_t plane_stride = (size_t)(pk.rows_pad / 32) * pk.KS * 64;
             v4i *P = (v4i *)pk.opnd + (size_t)b * planes * plane_stride;
-            for (uint32_t f = 0; f < nf; ++f)
-                for (uint32_t q = 0; q < nq; ++q) {
-                    const uint32_t sym = f * 4 + q, r = f * num_rot + q * nrr + i;
-                    const uint32_t *so = pk.symoff + (size_t)sym * pk.Epad;
-                    long long sq = 0;
-                    for (uint32_t piece = threadIdx.x; piece < pk.KS * 2; piece += blockDim.x) {
-                        v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
-                        const uint4 *so4 = (const uint4 *)(so + piece * 16);
+            const uint32_t pieces = pk.KS * 2, nsym = nf * nq;
+            auto clamp_q = [&](uint32_t po) {
+                const float v = fminf(fmaxf(__fmul_rn(s_base[po], factor), 0.0f), factor);   // NaN -> 0
+                return (uint32_t)v;
+            };
+            for (uint32_t item = threadIdx.x; item < nsym * pieces; item += blockDim.x) {
+                const uint32_t si = item / pieces, piece = item % pieces;
+                const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q, r = f * num_rot + q * nrr + i;
+                const uint4 *so4 = (const uint4 *)(pk.symoff + (size_t)sym * pk.Epad + piece * 16);
+                v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+                int hh = 0, hl = 0, ll = 0;
 #pragma unroll
-                        for (int w4 = 0; w4 < 4; ++w4) {
-                            const uint4 pv = so4[w4];
-                            const uint32_t pp[4] = {pv.x, pv.y, pv.z, pv.w};
-#pragma unroll
-                            for (int u = 0; u < 4; ++u) {
-                                if (piece * 16 + w4 * 4 + u < pk.E) {
-                                    const int qv = quantise(s_base[pp[u] & 0xffffffu], factor);
-                                    int h, l = 0;
-                                    if (U16) {
-                                        const int cv = qv - 32768;
-                                        h = cv >> 8;
-                                        l = (cv & 255) - 128;
-                                    } else {
-                                        h = qv - 128;
-                                    }
-                                    const long long v = U16 ? 256 * h + l : h;
-                                    sq += v * v;
-                                    hi[w4] |= (h & 255) << (8 * u);
-                                    lo[w4] |= (l & 255) << (8 * u);
-                                }
-                            }
-                        }
-                        const size_t frag = ((size_t)(r >> 5) * pk.KS + (piece >> 1)) * 64 + (r & 31) + 32 * (piece & 1);
-                        P[frag] = hi;
-                        if (U16) P[plane_stride + frag] = lo;
+                for (int w4 = 0; w4 < 4; ++w4) {
+                    const uint4 pv = so4[w4];
+                    const uint32_t k0 = piece * 16 + w4 * 4;
+                    const uint32_t valid = pk.E > k0 ? min(pk.E - k0, 4u) : 0u;
+                    const uint32_t live = valid >= 4 ? 0xffffffffu : (1u << (8 * valid)) - 1u;
+                    const uint32_t q0 = clamp_q(pv.x), q1 = clamp_q(pv.y), q2 = clamp_q(pv.z), q3 = clamp_q(pv.w);
+                    if constexpr (U16) {
+                        const uint32_t w01 = q0 | (q1 << 16), w23 = q2 | (q3 << 16);
+                        const int h = (int)((__builtin_amdgcn_perm(w23, w01, 0x07050301u) ^ 0x80808080u) & live);
+                        const int l = (int)((__builtin_amdgcn_perm(w23, w01, 0x06040200u) ^ 0x80808080u) & live);
+                        hi[w4] = h; lo[w4] = l;
+                        hh = __builtin_amdgcn_sdot4(h, h, hh, false);
+                        hl = __builtin_amdgcn_sdot4(h, l, hl, false);
+                        ll = __builtin_amdgcn_sdot4(l, l, ll, false);
+                    } else {
+                        const int h = (int)(((q0 | (q1 << 8) | (q2 << 16) | (q3 << 24)) ^ 0x80808080u) & live);
+                        hi[w4] = h;
+                        hh = __builtin_amdgcn_sdot4(h, h, hh, false);
                     }
-#pragma unroll
-                    for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
-                    if ((threadIdx.x & 63) == 0) atomicAdd(&s_norm[sym], (unsigned long long)sq);
                 }
+                const size_t frag = ((size_t)(r >> 5) * pk.KS + (piece >> 1)) * 64 + (r & 31) + 32 * (piece & 1);
+                P[frag] = hi;
+                if (U16) P[plane_stride + frag] = lo;
+                const long long sq = U16 ? ((long long)hh << 16) + (long long)hl * 512 + ll : (long long)hh;
+                if (sq) atomicAdd(&s_norm[sym], (unsigned long long)sq);
+            }
             __syncthreads();
             if (threadIdx.x < 8) {
                 const uint32_t f = threadIdx.x >> 2, q = threadIdx.x & 3;
@@ -1121,6 +1125,10 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
     const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->D * sizeof(float) : 0;
+    // about four neuron pixels per thread: large neurons get large blocks, whose many waves per LDS
+    // footprint hide the latency of the gathers (measured: 1024 threads 35 % faster than 256 at 3 x 70 x 70)
+    uint32_t threads = 256;
+    while (threads < 1024 && threads * 4 < ctx->D * ctx->D) threads *= 2;
     PackArgs pk{};
     int pack = 0;
     if (ctx->fused_pack) {
@@ -1136,7 +1144,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
         }
     }
 #define LAUNCH_ROTATE(P_)                                                                                          \
-    hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(256), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
+    hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
                        ctx->use_lds ? 1u : 0u, pk)
     switch (pack) {
