@@ -1514,10 +1514,11 @@ int init_ctx(pink_hip_ctx *ctx)
             ctx->Np = round_up(ctx->N, 64);
             ctx->Rp = round_up(ctx->R, 64);
             const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
-            // k is cut so that every CU gets about two waves; a block of four waves takes one slice
-            uint32_t cuts = std::max(1u, (2u * (uint32_t)ctx->num_cu + tiles - 1) / tiles);
-            cuts = std::min(cuts, std::max(1u, ctx->gKS / 4));
-            uint32_t slices = (cuts + 3) / 4;
+            // k is cut into as many slices as keep all blocks (one per tile and slice, four waves each)
+            // resident at once, one per CU, with at least four k-steps per wave (measured at 72 tiles:
+            // 3 slices = 216 blocks beat 2 by 4 % and 4, a second round of blocks, by 30 %)
+            uint32_t slices = std::max(1u, (uint32_t)ctx->num_cu / tiles);
+            slices = std::min(slices, std::max(1u, ctx->gKS / 16));
             // few k-steps per wave either way: one block per tile, which then finishes the tile itself
             if ((ctx->gKS + 3) / 4 <= 8) slices = 1;
             ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
