@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define PINK_HIP_ABI_VERSION 1
+#define PINK_HIP_ABI_VERSION 2
 
 typedef enum pink_hip_status {
     PINK_HIP_OK = 0,
@@ -112,9 +112,17 @@ int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som);
 /* Trainer<...,true>::operator()(Data const&) (Trainer.h:263-304) applied to n_images
  * images in order with sequential SOM semantics (image k+1 sees the weights left by
  * image k, Pink/main_generic.h:87-89); n_images = 1 is exactly one operator() call.
- * bmu_out (may be NULL) receives the best-matching neuron of each image, which the
- * caller adds to m_update_info (Trainer.h:302-303). */
+ * bmu_out receives the best-matching neuron of each image, which the caller adds to
+ * m_update_info (Trainer.h:302-303); the call then returns when they are there.
+ * With bmu_out NULL and up to 128 KiB of images the call copies the images and returns
+ * with the work queued on the context's stream (operator() returns nothing either): a
+ * loop of per-image calls then runs at the rate of the kernels, not of the round trips.
+ * pink_hip_get_som, pink_hip_update_counts and pink_hip_synchronize wait for queued work;
+ * an error of queued work is reported by the next call that waits. */
 int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out);
+/* m_update_info (Trainer.h:79,94-95,302-303): how often each of the N neurons was the
+ * best match, over all images this context has trained, counted on the device. */
+int pink_hip_update_counts(pink_hip_ctx *ctx, uint32_t *host_counts_out);
 /* Same with the images already on the device and the BMUs left on the device;
  * asynchronous on the context's stream (see pink_hip_synchronize). */
 int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, uint32_t *dev_bmu_out);

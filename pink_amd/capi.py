@@ -29,7 +29,7 @@ EXPORTS = (
     "pink_hip_distance", "pink_hip_region_size", "pink_hip_distance_kernel", "pink_hip_set_profiling",
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
     "pink_hip_make_update_factors", "pink_hip_layout_distances", "pink_hip_shuffled_order",
-    "pink_hip_fill_random_uniform",
+    "pink_hip_fill_random_uniform", "pink_hip_update_counts",
 )
 
 
@@ -69,6 +69,7 @@ def lib():
         L.pink_hip_set_som.argtypes = [vp, f32p]
         L.pink_hip_get_som.argtypes = [vp, f32p]
         L.pink_hip_train.argtypes = [vp, f32p, u32, u32p]
+        L.pink_hip_update_counts.argtypes = [vp, u32p]
         L.pink_hip_train_device.argtypes = [vp, vp, u32, vp]
         L.pink_hip_map.argtypes = [vp, f32p, u32, f32p, u32p]
         L.pink_hip_map_device.argtypes = [vp, vp, u32, vp, vp]
@@ -223,13 +224,24 @@ class Context:
         self._check(self._L.pink_hip_get_som(self._h, _f32(out)))
         return out
 
-    def train(self, images):
+    def train(self, images, want_bmu=True):
+        """Train on the images in order.  want_bmu=False returns nothing and, for up to 128 KiB of
+        images, does not wait for the GPU (see update_counts / synchronize / get_som)."""
         images = np.ascontiguousarray(images, np.float32)
         n = images.size // self.image_size
         assert n * self.image_size == images.size
+        if not want_bmu:
+            self._check(self._L.pink_hip_train(self._h, _f32(images), n, None))
+            return None
         bmu = np.empty(n, np.uint32)
         self._check(self._L.pink_hip_train(self._h, _f32(images), n, _u32(bmu)))
         return bmu
+
+    def update_counts(self):
+        """How often each neuron was the best match so far (the reference's update info)."""
+        counts = np.empty(self.N, np.uint32)
+        self._check(self._L.pink_hip_update_counts(self._h, _u32(counts)))
+        return counts
 
     def train_device(self, dev_images_ptr, n, dev_bmu_ptr=None):
         self._check(self._L.pink_hip_train_device(self._h, dev_images_ptr, n, dev_bmu_ptr))

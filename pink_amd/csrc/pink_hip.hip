@@ -764,7 +764,8 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
                                                 const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
                                                 uint32_t N, uint32_t S, uint32_t parts, uint32_t shift,
                                                 void *__restrict__ somP, const uint32_t *__restrict__ inv,
-                                                uint32_t Epad, float qfactor, UpdatePlanes up)
+                                                uint32_t Epad, float qfactor, UpdatePlanes up,
+                                                uint32_t *__restrict__ counts)
 {
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
@@ -817,7 +818,10 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
     const uint32_t bmu = bi;
-    if (n == 0 && part == 0 && tid == 0) *bmu_out = bmu;
+    if (n == 0 && part == 0 && tid == 0) {
+        *bmu_out = bmu;
+        atomicAdd(&counts[bmu], 1u);           // m_update_info[bmu]++ (Trainer.h:302-303)
+    }
 
     const float f = factors[(size_t)bmu * N + n];
     if (f == 0.0f) {
@@ -944,7 +948,11 @@ struct pink_hip_ctx {
     float *st_img = nullptr, *st_heat = nullptr;
     uint32_t *st_best = nullptr, *st_bmu = nullptr;
     size_t st_images = 0;                  // capacity of the staging buffers, in images
-    char *st_pin = nullptr;                // kPinBytes in, kPinBytes out
+    char *st_pin = nullptr;                // kPinBytes in (as a whole, or as a ring of kPinSlots slots), kPinBytes out
+    hipEvent_t st_ev[8] = {};              // per slot: the copy out of it has run
+    uint32_t st_slot = 0;
+    bool st_ring_busy = false;             // a call returned with copies out of the ring still queued
+    uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
     bool fused_som = false;                // integer GEMM trainer: k_update refreshes the SOM planes and norms itself
@@ -1295,7 +1303,7 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
                        dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,
                        (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,
-                       is_int(ctx) ? (float)ctx->factor : 0.0f, up);
+                       is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts);
     if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
 }
@@ -1323,6 +1331,8 @@ int free_all(pink_hip_ctx *ctx)
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
+    for (hipEvent_t e : ctx->st_ev) if (e) (void)hipEventDestroy(e);
+    if (ctx->d_counts) (void)hipFree(ctx->d_counts);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
 }
@@ -1610,6 +1620,8 @@ int init_ctx(pink_hip_ctx *ctx)
         HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, symoff.data(), symoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
     }
     TRY(dev_alloc(ctx, &ctx->d_bmu_scratch, 1));
+    TRY(dev_alloc(ctx, &ctx->d_counts, ctx->N));
+    HIP_TRY(ctx, hipMemset(ctx->d_counts, 0, (size_t)ctx->N * sizeof(uint32_t)));
     TRY(dev_alloc(ctx, &ctx->d_dist, B * ctx->N));
     TRY(dev_alloc(ctx, &ctx->d_ssd, B * ctx->N));
     TRY(dev_alloc(ctx, &ctx->d_best, B * ctx->N));
@@ -1807,6 +1819,16 @@ int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som)
     return PINK_HIP_OK;
 }
 
+int pink_hip_update_counts(pink_hip_ctx *ctx, uint32_t *host_counts_out)
+{
+    if (!ctx || !host_counts_out) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_update_counts: null argument");
+    if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_update_counts: context was created without update factors");
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, hipMemcpyAsync(host_counts_out, ctx->d_counts, (size_t)ctx->N * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return PINK_HIP_OK;
+}
+
 int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, uint32_t *dev_bmu_out)
 {
     if (!ctx || (!dev_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train_device: null argument");
@@ -1828,6 +1850,8 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
 }
 
 constexpr size_t kPinBytes = (size_t)1 << 20;
+constexpr uint32_t kPinSlots = 8;
+constexpr size_t kSlotBytes = kPinBytes / kPinSlots;
 
 // Staging for `n` images per chunk (grown on demand, freed with the context).
 int ensure_staging(pink_hip_ctx *ctx, size_t n)
@@ -1837,6 +1861,7 @@ int ensure_staging(pink_hip_ctx *ctx, size_t n)
             ctx->st_pin = nullptr;
             return fail(ctx, PINK_HIP_ENOMEM, "pinned host allocation failed");
         }
+        for (hipEvent_t &e : ctx->st_ev) HIP_TRY(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
     }
     if (n <= ctx->st_images) return PINK_HIP_OK;
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -1859,6 +1884,11 @@ int ensure_staging(pink_hip_ctx *ctx, size_t n)
 hipError_t stage_in(pink_hip_ctx *ctx, void *dev, const void *host, size_t bytes)
 {
     if (bytes <= kPinBytes) {
+        if (ctx->st_ring_busy) {                           // queued calls may still read the buffer
+            const hipError_t e = hipStreamSynchronize(ctx->stream);
+            if (e != hipSuccess) return e;
+            ctx->st_ring_busy = false;
+        }
         memcpy(ctx->st_pin, host, bytes);
         return hipMemcpyAsync(dev, ctx->st_pin, bytes, hipMemcpyHostToDevice, ctx->stream);
     }
@@ -1871,8 +1901,23 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
     if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_train: context was created without update factors");
     if (n_images == 0) return PINK_HIP_OK;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    // Stage the images in chunks of at most ~1 GiB.
     const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
+    if (!host_bmu_out && n_images * img_bytes <= kSlotBytes) {
+        // Nothing to hand back (the reference's operator() returns nothing either): the images are
+        // copied into a slot of the pinned ring and the call returns with the work queued, so a loop of
+        // per-image calls keeps the GPU busy instead of waiting for each image in turn.
+        TRY(ensure_staging(ctx, n_images));
+        const uint32_t slot = ctx->st_slot;
+        ctx->st_slot = (slot + 1) % kPinSlots;
+        HIP_TRY(ctx, hipEventSynchronize(ctx->st_ev[slot]));          // the copy that last used the slot has run
+        char *pin = ctx->st_pin + (size_t)slot * kSlotBytes;
+        memcpy(pin, host_images, n_images * img_bytes);
+        HIP_TRY(ctx, hipMemcpyAsync(ctx->st_img, pin, n_images * img_bytes, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(ctx, hipEventRecord(ctx->st_ev[slot], ctx->stream));
+        ctx->st_ring_busy = true;
+        return pink_hip_train_device(ctx, ctx->st_img, n_images, ctx->st_bmu);
+    }
+    // Stage the images in chunks of at most ~1 GiB.
     const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
     TRY(ensure_staging(ctx, chunk));
     for (uint32_t done = 0; done < n_images; done += chunk) {

@@ -104,8 +104,9 @@ public:
     {
         if (channels != m_cfg.channels) throw pink::exception("image and neuron channel counts differ");
         if (m_ctx and image_dim == m_cfg.image_dim) return m_ctx;
-        if (m_ctx) {            // image size changed: keep the trained weights
+        if (m_ctx) {            // image size changed: keep the trained weights and the update counts
             check(m_ctx, pink_hip_get_som(m_ctx, m_som_copy.data()));
+            if (!m_factors.empty()) m_counts_base = update_counts();
             pink_hip_destroy(m_ctx);
             m_ctx = nullptr;
         }
@@ -119,6 +120,15 @@ public:
     }
 
     pink_hip_ctx* get() const { return m_ctx; }
+
+    /// How often each neuron was the best match, over every context this object has had.
+    std::vector<uint32_t> update_counts() const
+    {
+        std::vector<uint32_t> counts(m_cfg.som_size, 0u);
+        if (m_ctx) check(m_ctx, pink_hip_update_counts(m_ctx, counts.data()));
+        for (size_t i = 0; i < m_counts_base.size(); ++i) counts[i] += m_counts_base[i];
+        return counts;
+    }
     std::vector<float> const& initial_som() const { return m_som_copy; }
 
 private:
@@ -126,6 +136,7 @@ private:
     pink_hip_config m_cfg{};
     std::vector<float> m_factors;
     std::vector<float> m_som_copy;
+    std::vector<uint32_t> m_counts_base;
 };
 
 } // namespace hip_detail
@@ -148,8 +159,7 @@ public:
         EuclideanDistanceShape const& euclidean_distance_shape = EuclideanDistanceShape::QUADRATIC,
         [[maybe_unused]] uint32_t block_size = 256, DataType euclidean_distance_type = DataType::FLOAT)
      : m_som(som),
-       m_verbosity(verbosity),
-       m_update_info(som.get_som_layout(), 0u)
+       m_verbosity(verbosity)
     {
         if (number_of_rotations == 0 or (number_of_rotations != 1 and number_of_rotations % 4 != 0))
             throw pink::exception("Number of rotations must be 1 or larger then 1 and divisible by 4");
@@ -175,18 +185,15 @@ public:
         uint32_t channels = 0, image_dim = 0;
         hip_detail::image_geometry(data.get_layout(), channels, image_dim);
         auto* ctx = m_device.for_image(channels, image_dim);
-        uint32_t best_match = 0;
-        hip_detail::check(ctx, pink_hip_train(ctx, data.get_data_pointer(), 1, &best_match));
-        ++m_update_info[best_match];
+        // nothing is handed back: the library copies the image and returns with the work queued
+        hip_detail::check(ctx, pink_hip_train(ctx, data.get_data_pointer(), 1, nullptr));
     }
 
     /// Training by several data points stored back to back, in order
     void operator () (T const* images, uint32_t number_of_images, uint32_t channels, uint32_t image_dim)
     {
         auto* ctx = m_device.for_image(channels, image_dim);
-        std::vector<uint32_t> best_match(number_of_images);
-        hip_detail::check(ctx, pink_hip_train(ctx, images, number_of_images, best_match.data()));
-        for (auto b : best_match) ++m_update_info[b];
+        hip_detail::check(ctx, pink_hip_train(ctx, images, number_of_images, nullptr));
     }
 
     void update_som()
@@ -194,14 +201,20 @@ public:
         if (auto* ctx = m_device.get()) hip_detail::check(ctx, pink_hip_get_som(ctx, m_som.get_data_pointer()));
     }
 
-    auto get_update_info() const { return m_update_info; }
+    /// m_update_info of the reference (Trainer.h:79,94-95): counted on the device, read back here
+    auto get_update_info() const
+    {
+        UpdateInfoType info(m_som.get_som_layout(), 0u);
+        auto const counts = m_device.update_counts();
+        for (size_t i = 0; i < counts.size(); ++i) info[static_cast<uint32_t>(i)] = counts[i];
+        return info;
+    }
 
 private:
 
     /// A reference to the SOM will be trained
     SOMType& m_som;
     int m_verbosity;
-    UpdateInfoType m_update_info;
     hip_detail::Context m_device;
 };
 

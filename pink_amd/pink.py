@@ -188,6 +188,8 @@ class _Device:
                          interpolation=int(interpolation), update_factors=update_factors)
         self.ctx = None
         self.image_dim = None
+        self.update_factors = update_factors
+        self.counts_base = None
         # argument errors surface at construction, as in the reference: probe with the neuron size
         # (the library checks its arguments before it touches a device)
         try:
@@ -199,6 +201,11 @@ class _Device:
     def _context(self, image_dim):
         return capi.Context(self.som.number_of_neurons, self.channels, image_dim, self.neuron_dim, **self.args)
 
+    def update_counts(self):
+        """How often each neuron was the best match, over every context this object has had."""
+        counts = np.zeros(self.som.number_of_neurons, np.uint32) if self.ctx is None else self.ctx.update_counts()
+        return counts if self.counts_base is None else counts + self.counts_base
+
     def for_images(self, images, layout):
         images = np.ascontiguousarray(images, np.float32)
         per_image_ndim = 3 if self.channels > 1 or layout == "cartesian-3d" else 2
@@ -209,6 +216,8 @@ class _Device:
         if self.ctx is None or image_dim != self.image_dim:
             weights = self.ctx.get_som() if self.ctx is not None else self.som._rows()
             if self.ctx is not None:
+                if self.update_factors is not None:           # the counts of the context that goes away
+                    self.counts_base = self.update_counts()
                 self.ctx.close()
             self.ctx = self._context(image_dim)
             self.ctx.set_som(weights)
@@ -229,7 +238,6 @@ class Trainer:
         self._dev = _Device(som, number_of_rotations, use_flip, interpolation, use_gpu, euclidean_distance_dim,
                             euclidean_distance_shape, euclidean_distance_type, self.update_factors)
         self._som = som
-        self.update_info = np.zeros(som.number_of_neurons, np.uint32)     # TrainerCommon::m_update_info
         self.verbosity = verbosity
 
     @staticmethod
@@ -248,20 +256,26 @@ class Trainer:
         return np.ascontiguousarray(factors, np.float32)
 
     def __call__(self, data):
-        """One image (Trainer.h:263-304)."""
-        self.train(np.asarray(data)[None], getattr(data, "layout", "cartesian-2d"))
+        """One image (Trainer.h:263-304).  Returns nothing, like the reference, and does not wait for
+        the GPU: the image is copied and the work queued; update_som() and get_update_info() wait."""
+        images = self._dev.for_images(np.asarray(data)[None], getattr(data, "layout", "cartesian-2d"))
+        self._dev.ctx.train(images, want_bmu=False)
 
     def train(self, images, layout="cartesian-2d"):
-        """Many images in order, one call: image k+1 sees the weights left by image k."""
+        """Many images in order, one call: image k+1 sees the weights left by image k.  Returns the
+        best-matching neuron of every image."""
         images = self._dev.for_images(images, layout)
-        bmu = self._dev.ctx.train(images)
-        np.add.at(self.update_info, bmu, 1)
-        return bmu
+        return self._dev.ctx.train(images)
 
     def update_som(self):
         """Device weights -> the SOM object (Trainer.h:306-309)."""
         if self._dev.ctx is not None:
             self._som._rows()[...] = self._dev.ctx.get_som()
+
+    @property
+    def update_info(self):
+        """TrainerCommon::m_update_info: how often each neuron was the best match (counted on the device)."""
+        return self._dev.update_counts()
 
     def get_update_info(self):
         return self.update_info

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(L, name), "libpink_hip.so does not export " + name
     assert declared == set(capi.EXPORTS)
-    assert L.pink_hip_abi_version() == 1
+    assert L.pink_hip_abi_version() == 2
 
 
 @pytest.mark.parametrize("num_rot", [0, 3, 90, 6])

@@ -159,3 +159,38 @@ def test_hexagonal_som_with_three_channels():
     s = O.shape(7, 2, 14, 10, 4, True, 6, O.QUADRATIC, capi.FLOAT)
     O.train(s, want, images, F)
     assert np.array_equal(np.array(som, copy=False).reshape(7, -1).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_per_image_calls_are_queued_and_counted_on_the_device():
+    # 40 operator() calls in a row (more than the ring of staging slots holds), a call that hands the
+    # best-matching neurons back in between, an image of another size (a new device context), and the
+    # update counts over all of it
+    rng = np.random.default_rng(3)
+    np_som = rng.random((3, 3, 10, 10), dtype=np.float32)
+    images = rng.random((45, 14, 14), dtype=np.float32)
+    som = pink.SOM(np_som.copy())
+    trainer = pink.Trainer(som, pink.GaussianFunctor(1.1, 0.2), number_of_rotations=4, use_flip=True,
+                           euclidean_distance_dim=6, euclidean_distance_type=pink.DataType.UINT8)
+    assert trainer.get_update_info().sum() == 0
+    for img in images[:20]:
+        trainer(pink.Data(img))
+    bmu_mid = trainer.train(images[20:25])
+    for img in images[25:]:
+        trainer(pink.Data(img))
+    F = capi.make_update_factors(capi.CARTESIAN, [3, 3], capi.GAUSSIAN, 1.1, 0.2)
+    want = np_som.reshape(9, -1).copy()
+    s = O.shape(9, 1, 14, 10, 4, True, 6, O.QUADRATIC, capi.UINT8)
+    obmu = O.train(s, want, images[:, None], F)
+    assert np.array_equal(bmu_mid, obmu[20:25])
+    assert np.array_equal(trainer.get_update_info(), np.bincount(obmu, minlength=9))
+    trainer.update_som()
+    assert np.array_equal(np.array(som, copy=False).reshape(9, -1).view(np.uint32), want.view(np.uint32))
+    # a larger image: the weights and the counts carry over into the new context
+    big = rng.random((1, 18, 18), dtype=np.float32)
+    trainer(pink.Data(big[0]))
+    s2 = O.shape(9, 1, 18, 10, 4, True, 6, O.QUADRATIC, capi.UINT8)
+    obmu2 = O.train(s2, want, big[:, None], F)
+    assert np.array_equal(trainer.get_update_info(), np.bincount(np.concatenate([obmu, obmu2]), minlength=9))
+    trainer.update_som()
+    assert np.array_equal(np.array(som, copy=False).reshape(9, -1).view(np.uint32), want.view(np.uint32))
