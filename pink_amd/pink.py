@@ -75,6 +75,15 @@ class GaussianFunctor:
         return float(d / (s * np.sqrt(np.float32(2.0) * np.float32(math.pi))) * np.exp(np.float32(-0.5) * x * x))
 
 
+class LibraryFunctor:
+    """A neighbourhood function of UtilitiesLib/DistributionFunctor.cpp:19-59 by kind (capi.STEP, GAUSSIAN,
+    UNITY_GAUSSIAN, MEXICAN_HAT): the library evaluates it with the reference's float arithmetic.  Not in
+    the reference's Python module (which exports GaussianFunctor only); the command line selects them."""
+
+    def __init__(self, kind, sigma, damping):
+        self.kind, self.sigma, self.damping = int(kind), float(sigma), float(damping)
+
+
 def _as_float32_copy(buffer, what):
     a = np.asarray(buffer)
     if a.dtype != np.float32:
@@ -244,9 +253,10 @@ class Trainer:
     def _update_factors(som, function, max_update_distance):
         """TrainerCommon's constructor loop (Trainer.h:69-76): f(distance) where the distance is
         below max_update_distance (or that is not positive), else 0."""
-        if type(function) is GaussianFunctor:
-            # the library evaluates this functor itself, with the reference's float arithmetic
-            return capi.make_update_factors(som._layout, som._dims, capi.GAUSSIAN, function.sigma, function.damping,
+        if type(function) in (GaussianFunctor, LibraryFunctor):
+            # the library evaluates these functors itself, with the reference's float arithmetic
+            kind = capi.GAUSSIAN if type(function) is GaussianFunctor else function.kind
+            return capi.make_update_factors(som._layout, som._dims, kind, function.sigma, function.damping,
                                             max_update_distance)
         dist = capi.layout_distances(som._layout, som._dims)
         values = {float(d): np.float32(function(float(d))) for d in np.unique(dist)}
