@@ -10,8 +10,11 @@
 
 namespace pink_sym {
 
-// Once per context: allow the rotation kernel its LDS images (C x (I+1) x (I+1) floats each) and
-// the distance kernel of this KS (8, 16, 24 or 32 k-steps) its three LDS buffers.
+// LDS bytes of one image in the rotation kernel (padded rows).
+size_t lds_image_bytes(uint32_t C, uint32_t I);
+
+// Once per context: allow the rotation kernel its LDS images (lds_image_bytes each) and the
+// distance kernel of this KS (8, 16, 24 or 32 k-steps) its three LDS buffers.
 hipError_t configure(uint32_t KS, uint32_t C, uint32_t I);
 
 // The geometry of the base rotations (source offset and bilinear weights per rotation and union

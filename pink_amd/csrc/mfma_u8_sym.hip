@@ -41,6 +41,19 @@ __device__ __forceinline__ int32_t quantise(float x, float factor)
     return (int32_t)v;
 }
 
+// Row stride (floats) of an image in the rotation kernel's LDS: the I pixels, at least one zero
+// column, and congruent to 5 modulo 8.  The banks of the four neighbours of a rotated position
+// are (stride * row + column) mod 64; the lanes of a wave read the same position under 32
+// neighbouring angles, i.e. a short arc of texels, and with stride = 1 mod 64 (I = 64 with a single
+// pad column) every arc along the anti-diagonal would stay in one bank (measured at I = 64: strides 67 to 73
+// are 19 % faster than 65).
+inline uint32_t row_stride(uint32_t I)
+{
+    uint32_t W = I + 1;
+    while (W % 8 != 5) ++W;
+    return W;
+}
+
 // SOM operand.  One block per row m = n * 8 + s (rows beyond 8 N are zero).
 // aoff[s][k] = neuron element paired with union position k under symmetry s, or ~0.
 __global__ __launch_bounds__(256) void k_pack_som_sym_u8(const float *__restrict__ som, const uint32_t *__restrict__ aoff,
@@ -87,12 +100,13 @@ __global__ __launch_bounds__(256) void k_pack_som_sym_u8(const float *__restrict
 __global__ __launch_bounds__(256) void k_rot_table(const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                    const uint32_t *__restrict__ upos, uint32_t Ku, uint32_t I,
                                                    uint32_t D, uint32_t nrr_eff, uint32_t Kp, uint32_t rows,
-                                                   uint32_t *__restrict__ tab_idx, float4 *__restrict__ tab_w)
+                                                   uint32_t W, uint32_t *__restrict__ tab_idx,
+                                                   float4 *__restrict__ tab_w)
 {
     const uint32_t t = blockIdx.x * 256 + threadIdx.x;
     if (t >= rows * Kp) return;
     const uint32_t i = t / Kp, k = t % Kp;
-    const uint32_t W = I + 1, CH = W * W;
+    const uint32_t CH = (I + 1) * W;                      // W = row stride of the LDS image
     uint32_t idx = I;                                     // row 0 of the extra column: 0.0
     float4 w = {0.0f, 0.0f, 0.0f, 0.0f};
     if (i < nrr_eff && k < Ku) {
@@ -152,9 +166,9 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
                                                         const float4 *__restrict__ tab_w,
                                                         const unsigned char *__restrict__ kmask, uint32_t Ku,
                                                         uint32_t all_sym, uint32_t C, uint32_t I, uint32_t nrr_eff,
-                                                        uint32_t KS, uint32_t RTP, uint32_t B)
+                                                        uint32_t KS, uint32_t RTP, uint32_t B, uint32_t W)
 {
-    extern __shared__ float s_img[];                      // G x C x (I + 1) x (I + 1), zero padded
+    extern __shared__ float s_img[];                      // G x C x (I + 1) rows of row_stride(I), zero padded
     __shared__ int s_nb[G][32][8];
     const uint32_t UNIT_V = KS * 64 + 64;                 // 16-byte vectors per unit: fragments, then norm entries
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The
@@ -166,7 +180,7 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
     const uint32_t b0 = ((lin / span) * 8 + (lin % 8)) * G;
     if (b0 >= B) return;
     const uint32_t ng = min((uint32_t)G, B - b0);
-    const uint32_t W = I + 1, CH = W * W, II = I * I, IMG = C * CH;
+    const uint32_t CH = (I + 1) * W, II = I * I, IMG = C * CH;
     const uint32_t nthreads = blockDim.x;
     for (uint32_t t = threadIdx.x; t < G * 32 * 8; t += nthreads) (&s_nb[0][0][0])[t] = 0;
     // Copy the batch into the padded tiles.  The loads of up to 8 elements per thread are issued
@@ -213,9 +227,9 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
                 }
             }
         }
-        for (uint32_t t = threadIdx.x; t < ng * C * W; t += nthreads) {
-            const uint32_t gc = t / W, r = t % W;
-            s_img[gc * CH + r * W + I] = 0.0f;            // extra column
+        for (uint32_t t = threadIdx.x; t < ng * C * (I + 1); t += nthreads) {
+            const uint32_t gc = t / (I + 1), r = t % (I + 1);
+            s_img[gc * CH + r * W + I] = 0.0f;            // extra column (the only pad column ever read)
             s_img[gc * CH + I * W + r] = 0.0f;            // extra row
         }
     }
@@ -556,30 +570,33 @@ hipError_t pack_som(hipStream_t stream, const float *som, const uint32_t *aoff, 
     return hipGetLastError();
 }
 
+size_t lds_image_bytes(uint32_t C, uint32_t I) { return (size_t)C * (I + 1) * row_stride(I) * sizeof(float); }
+
 // images per block of the rotation kernel: as many as let two blocks share a CU's LDS (one loads
 // its images while the other computes), next to their norm counters
-uint32_t images_per_block(size_t lds_image_bytes)
+uint32_t images_per_block(size_t image_bytes)
 {
-    const size_t budget = 72 * 1024;
-    return lds_image_bytes * 4 <= budget ? 4 : lds_image_bytes * 2 <= budget ? 2 : 1;
+    const size_t budget = 76 * 1024;                      // two blocks and their counters within 160 KiB
+    return image_bytes * 4 <= budget ? 4 : image_bytes * 2 <= budget ? 2 : 1;
 }
 
 template <int G>
 hipError_t launch_rotpack(hipStream_t stream, const RotpackArgs &g, bool configure_only)
 {
-    const size_t lds = (size_t)G * g.C * (g.I + 1) * (g.I + 1) * sizeof(float);
+    const size_t lds = (size_t)G * lds_image_bytes(g.C, g.I);
     if (configure_only)
         return hipFuncSetAttribute((const void *)k_rotpack_sym_u8<G>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     const uint32_t groups = (g.B + G - 1) / G;
     const uint32_t blocks = ((groups + 7) / 8) * 8 * g.RTP;           // 8 groups per span of ids, see the kernel
     hipLaunchKernelGGL(k_rotpack_sym_u8<G>, dim3(blocks), dim3(G >= 4 ? 512 : 256), lds, stream, g.images, (v4i *)g.Pb, g.tab_idx,
-                       (const float4 *)g.tab_w, g.kmask, g.Ku, g.all_sym, g.C, g.I, g.nrr_eff, g.KS, g.RTP, g.B);
+                       (const float4 *)g.tab_w, g.kmask, g.Ku, g.all_sym, g.C, g.I, g.nrr_eff, g.KS, g.RTP, g.B,
+                       row_stride(g.I));
     return hipGetLastError();
 }
 
 hipError_t dispatch_rotpack(hipStream_t stream, const RotpackArgs &g, bool configure_only)
 {
-    switch (images_per_block((size_t)g.C * (g.I + 1) * (g.I + 1) * sizeof(float))) {
+    switch (images_per_block(lds_image_bytes(g.C, g.I))) {
     case 4: return launch_rotpack<4>(stream, g, configure_only);
     case 2: return launch_rotpack<2>(stream, g, configure_only);
     default: return launch_rotpack<1>(stream, g, configure_only);
@@ -606,7 +623,7 @@ hipError_t build_rot_table(hipStream_t stream, const float *cos_t, const float *
     float4 *tab_w = (float4 *)table;                                   // weights first: 16-byte aligned
     uint32_t *tab_idx = (uint32_t *)(tab_w + (size_t)rows * Kp);
     hipLaunchKernelGGL(k_rot_table, dim3((rows * Kp + 255) / 256), dim3(256), 0, stream, cos_t, sin_t, upos, Ku, I, D, nrr_eff,
-                       Kp, rows, tab_idx, tab_w);
+                       Kp, rows, row_stride(I), tab_idx, tab_w);
     return hipGetLastError();
 }
 

@@ -137,8 +137,10 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
-                                                uint32_t use_flip, uint32_t use_lds, PackArgs pk)
+                                                uint32_t use_flip, uint32_t use_lds, uint32_t Dp, PackArgs pk)
 {
+    // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
+    // stride keeps those reads in different banks (a stride of 64 would put all of them into one)
     extern __shared__ float s_base[];
     __shared__ unsigned long long s_norm[8];
     const uint32_t i = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
 
     if (use_lds) {
         for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x)
-            s_base[p] = base_pixel(img, I, D, i, cs, sn, p / D, p % D);
+            s_base[(p / D) * Dp + p % D] = base_pixel(img, I, D, i, cs, sn, p / D, p % D);
         __syncthreads();
         for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
             const uint32_t x = p / D, y = p % D;
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     default: a = y; bb = D - 1 - xs; break;
                     }
                     const uint32_t k = f * num_rot + q * nrr + i;
-                    out[((size_t)k * C + c) * DD + p] = s_base[a * D + bb];
+                    out[((size_t)k * C + c) * DD + p] = s_base[a * Dp + bb];
                 }
             }
         }
@@ -918,6 +920,7 @@ struct pink_hip_ctx {
     uint32_t N = 0, C = 0, I = 0, D = 0, S = 0, R = 0, nrr = 0, E = 0, Epad = 0, Rpad = 0;
     uint32_t isz = 0;          // floats per image
     uint32_t Bcap = 1;         // images per launch group
+    uint32_t Dp = 0;           // row stride of the rotation kernel's LDS tile
     uint32_t shift = 32;       // key = value << shift | rotation
     uint32_t factor = 1;       // 255 / 65535 in the integer modes
     bool trainer = false;
@@ -1132,7 +1135,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 {
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
-    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->D * sizeof(float) : 0;
+    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->Dp * sizeof(float) : 0;
     // about four neuron pixels per thread: large neurons get large blocks, whose many waves per LDS
     // footprint hide the latency of the gathers (measured: 1024 threads 35 % faster than 256 at 3 x 70 x 70)
     uint32_t threads = 256;
@@ -1154,7 +1157,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 #define LAUNCH_ROTATE(P_)                                                                                          \
     hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
-                       ctx->use_lds ? 1u : 0u, pk)
+                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
     case 2: LAUNCH_ROTATE(2); break;
@@ -1435,7 +1438,7 @@ int init_ctx(pink_hip_ctx *ctx)
             std::vector<char> seen(ctx->S, 0);
             for (uint32_t e = 0; e < ctx->E; ++e) { if (seen[region[e]]) distinct = false; seen[region[e]] = 1; }
         }
-        const size_t lds_img = (size_t)ctx->C * (ctx->I + 1) * (ctx->I + 1) * sizeof(float);
+        const size_t lds_img = pink_sym::lds_image_bytes(ctx->C, ctx->I);
         const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 32 && ctx->RTP <= 3 &&
                               lds_img <= 150 * 1024 && D < 4096 && ctx->C < 256;
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM && !fits_sym)
@@ -1556,7 +1559,8 @@ int init_ctx(pink_hip_ctx *ctx)
         ctx->Bcap = (uint32_t)b;
     }
     const size_t B = ctx->Bcap;
-    ctx->use_lds = (size_t)ctx->D * ctx->D * sizeof(float) <= 64 * 1024;
+    ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
+    ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= 64 * 1024;
 
     TRY(dev_alloc(ctx, &ctx->d_som, (size_t)ctx->N * ctx->S));
     HIP_TRY(ctx, hipMemset(ctx->d_som, 0, (size_t)ctx->N * ctx->S * sizeof(float)));
@@ -1613,7 +1617,7 @@ int init_ctx(pink_hip_ctx *ctx)
                 case 2: a = D - 1 - xs; bb = D - 1 - y; break;
                 default: a = y; bb = D - 1 - xs; break;
                 }
-                symoff[(size_t)sym * ctx->Epad + e] = (ch << 24) | (a * D + bb);
+                symoff[(size_t)sym * ctx->Epad + e] = (ch << 24) | (a * ctx->Dp + bb);     // LDS rows of Dp floats
             }
         }
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));

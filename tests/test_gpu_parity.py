@@ -260,6 +260,9 @@ FUSED_TRAIN_SHAPES = [
     (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.FLOAT, 4),        # three channels, float32 rows from the rotation kernel
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.FLOAT, 3),           # region repeats channel 0 (CPU rule): no inverse table
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.UINT16, 3),
+    (4, 1, 200, 150, 8, True, 100, capi.CIRCULAR, capi.UINT8, 2),     # neurons too large for the rotation kernel's LDS tile
+    (3, 1, 160, 129, 4, True, 128, capi.QUADRATIC, capi.FLOAT, 2),
+    (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
 ]
 
 
