@@ -147,6 +147,27 @@ __global__ __launch_bounds__(256) void k_rot_table(const float *__restrict__ cos
     tab_idx[(((size_t)piece * 4 + j / 4) * rows + i) * 4 + j % 4] = idx;
 }
 
+// Quotient and remainder by a divisor that is the same for the whole block, for dividends below
+// 2^24 (element counts of an LDS tile): a shift and a mask for a power of two, else the float
+// reciprocal's estimate, which is within one of the quotient, corrected.  The compiler's general
+// 32-bit division costs about four times as many instructions.
+struct BlockDivisor {
+    uint32_t d, mask;
+    int shift;              // >= 0: d = 1 << shift
+    float rcp;
+    __device__ explicit BlockDivisor(uint32_t d_) : d(d_), mask(d_ - 1), shift((d_ & (d_ - 1)) == 0 ? __builtin_ctz(d_) : -1),
+                                                    rcp(1.0f / (float)d_) {}
+    __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
+    {
+        if (shift >= 0) { q = n >> shift; r = n & mask; return; }
+        uint32_t e = (uint32_t)((float)n * rcp);
+        int rem = (int)(n - e * d);
+        if (rem < 0) { --e; rem += (int)d; }
+        else if ((uint32_t)rem >= d) { ++e; rem -= (int)d; }
+        q = e; r = (uint32_t)rem;
+    }
+};
+
 // Byte `byte` of `word` = q = uint8(x * 255), truncated and saturated to [0, 255] (NaN -> 0):
 // multiply, truncate, then the saturating convert-and-pack (which alone would round to nearest).
 __device__ __forceinline__ uint32_t pack_quantised_u8(float x, uint32_t byte, uint32_t word)
@@ -168,7 +189,9 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
                                                         uint32_t all_sym, uint32_t C, uint32_t I, uint32_t nrr_eff,
                                                         uint32_t KS, uint32_t RTP, uint32_t B, uint32_t W)
 {
-    extern __shared__ float s_img[];                      // G x C x (I + 1) rows of row_stride(I), zero padded
+    // C x (I + 1) rows of W pixels, zero padded, the G images interleaved per pixel: the four
+    // neighbours of a position are four reads of G floats for all images, from one address
+    extern __shared__ float s_img[];
     __shared__ int s_nb[G][32][8];
     const uint32_t UNIT_V = KS * 64 + 64;                 // 16-byte vectors per unit: fragments, then norm entries
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The
@@ -180,7 +203,7 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
     const uint32_t b0 = ((lin / span) * 8 + (lin % 8)) * G;
     if (b0 >= B) return;
     const uint32_t ng = min((uint32_t)G, B - b0);
-    const uint32_t CH = (I + 1) * W, II = I * I, IMG = C * CH;
+    const uint32_t CH = (I + 1) * W, II = I * I;
     const uint32_t nthreads = blockDim.x;
     for (uint32_t t = threadIdx.x; t < G * 32 * 8; t += nthreads) (&s_nb[0][0][0])[t] = 0;
     // Copy the batch into the padded tiles.  The loads of up to 8 elements per thread are issued
@@ -188,6 +211,7 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
     {
         const float *src = images + (size_t)b0 * C * II;
         const uint32_t total = ng * C * II;
+        const BlockDivisor by_II(II), by_I(I), by_C(C), by_rows(I + 1), by_G(G);
         if ((I & 3) == 0) {
             // rows are whole float4s: 16-byte loads, one division per vector
             const float4 *src4 = (const float4 *)src;
@@ -203,9 +227,12 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t e = base + j * nthreads + threadIdx.x;
                     if (e < total4) {
-                        const uint32_t gc = (4 * e) / II, rem = (4 * e) % II;
-                        float *d = s_img + gc * CH + (rem / I) * W + rem % I;
-                        d[0] = v[j].x; d[1] = v[j].y; d[2] = v[j].z; d[3] = v[j].w;
+                        uint32_t gc, rem, row, col, gi, c;
+                        by_II.divmod(4 * e, gc, rem);
+                        by_I.divmod(rem, row, col);
+                        by_C.divmod(gc, gi, c);
+                        float *d = s_img + (c * CH + row * W + col) * G + gi;
+                        d[0] = v[j].x; d[G] = v[j].y; d[2 * G] = v[j].z; d[3 * G] = v[j].w;
                     }
                 }
             }
@@ -221,16 +248,21 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t e = base + j * nthreads + threadIdx.x;
                     if (e < total) {
-                        const uint32_t gc = e / II, rem = e % II;
-                        s_img[gc * CH + (rem / I) * W + rem % I] = v[j];
+                        uint32_t gc, rem, row, col, gi, c;
+                        by_II.divmod(e, gc, rem);
+                        by_I.divmod(rem, row, col);
+                        by_C.divmod(gc, gi, c);
+                        s_img[(c * CH + row * W + col) * G + gi] = v[j];
                     }
                 }
             }
         }
-        for (uint32_t t = threadIdx.x; t < ng * C * (I + 1); t += nthreads) {
-            const uint32_t gc = t / (I + 1), r = t % (I + 1);
-            s_img[gc * CH + r * W + I] = 0.0f;            // extra column (the only pad column ever read)
-            s_img[gc * CH + I * W + r] = 0.0f;            // extra row
+        for (uint32_t t = threadIdx.x; t < G * C * (I + 1); t += nthreads) {
+            uint32_t gi, p, c, r;
+            by_G.divmod(t, p, gi);
+            by_rows.divmod(p, c, r);
+            s_img[(c * CH + r * W + I) * G + gi] = 0.0f;  // extra column (the only pad column ever read)
+            s_img[(c * CH + I * W + r) * G + gi] = 0.0f;  // extra row
         }
     }
     __syncthreads();
@@ -248,7 +280,12 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
         for (int gi = 0; gi < G; ++gi)
 #pragma unroll
             for (int w4 = 0; w4 < 4; ++w4) word[gi][w4] = 0;
-        uint32_t live[4] = {0, 0, 0, 0};
+        uint32_t live[4];                                 // byte masks of the positions inside the union
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            const int inside = (int)Ku - (int)(k0 + 4 * w4);
+            live[w4] = inside >= 4 ? 0xffffffffu : inside <= 0 ? 0u : (1u << (8 * inside)) - 1u;
+        }
         if (i < nrr_eff) {
             const uint4 *ti = (const uint4 *)tab_idx + (size_t)piece * 4 * rows + i;
             const float4 *tw = tab_w + (size_t)piece * 16 * rows + i;
@@ -259,17 +296,25 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const float4 wv = tw[(4 * w4 + u) * rows];
-                    const float *tap = s_img + ii[u];
-                    live[w4] |= (k0 + 4 * w4 + u < Ku ? 0xffu : 0u) << (8 * u);
+                    typedef float vecG __attribute__((ext_vector_type(G)));
+                    const float *tap = s_img + ii[u] * G;
                     // (all G images, also past the end of the batch: what is computed from LDS nobody
                     // filled is dropped below, and the loop stays free of branches)
+                    float t00[G], t01[G], t10[G], t11[G];
+                    if constexpr (G > 1) {
+                        const vecG a = *(const vecG *)tap, b = *(const vecG *)(tap + G);
+                        const vecG c = *(const vecG *)(tap + W * G), d = *(const vecG *)(tap + W * G + G);
+#pragma unroll
+                        for (int gi = 0; gi < G; ++gi) { t00[gi] = a[gi]; t01[gi] = b[gi]; t10[gi] = c[gi]; t11[gi] = d[gi]; }
+                    } else {
+                        t00[0] = tap[0]; t01[0] = tap[1]; t10[0] = tap[W]; t11[0] = tap[W + 1];
+                    }
 #pragma unroll
                     for (int gi = 0; gi < G; ++gi) {
-                        const float *tp = tap + gi * IMG;
-                        const float a = __fmul_rn(wv.x, tp[0]);
-                        const float b = __fmul_rn(wv.y, tp[1]);
-                        const float c = __fmul_rn(wv.z, tp[W]);
-                        const float d = __fmul_rn(wv.w, tp[W + 1]);
+                        const float a = __fmul_rn(wv.x, t00[gi]);
+                        const float b = __fmul_rn(wv.y, t01[gi]);
+                        const float c = __fmul_rn(wv.z, t10[gi]);
+                        const float d = __fmul_rn(wv.w, t11[gi]);
                         const float v = __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
                         word[gi][w4] = pack_quantised_u8(v, u, word[gi][w4]);
                     }
