@@ -448,12 +448,16 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     __syncthreads();
 
     // maximum over the 16 lanes that hold one neuron: the 8 symmetry lanes (two quad exchanges and
-    // a mirror of the half row, all in the data-parallel path) and the other half-wave
+    // a mirror of the half row, all in the data-parallel path) and the other half-wave (v_permlane32_swap:
+    // no trip through LDS)
     auto max16 = [&](int v) -> int {
         v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));    // lane ^ 1
         v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));    // lane ^ 2
         v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));   // 7 - lane in the half row
-        return max(v, __shfl_xor(v, 32, 64));
+        // the other half-wave: one swap of the upper half of one copy with the lower half of another
+        // leaves the lower half's value in all lanes of the first and the upper half's in the second
+        const auto halves = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+        return max((int)halves[0], (int)halves[1]);
     };
 
     // Bookkeeping.  The unit's norm entry of row j of this lane is  cj = (15 - j) - 16 |b_row|^2, so
@@ -464,6 +468,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     // rotation carry |b|^2 = 2^26 and never win.
     int m[2] = {INT_MIN, INT_MIN};
     uint32_t m_rt[2] = {0, 0};
+    uint32_t bk_rt = 0, bk_img = grp;                      // tile and image of the unit whose bookkeeping ends next
     auto finish_image = [&](uint32_t b) {
         // lexicographic minimum of (distance, variant) over the neuron's 16 lanes in two passes
 #pragma unroll
@@ -537,10 +542,11 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
         }
         if (src_u + 1 < nunits) advance_src();
         if (u > 0) {
-            const uint32_t rt = (u - 1) % RTP;
-            if (m[0] != m_before[0]) m_rt[0] = rt;
-            if (m[1] != m_before[1]) m_rt[1] = rt;
-            if (rt + 1 == RTP) finish_image(grp + ((u - 1) / RTP) * groups);
+            // (unit u - 1 = image bk_img, tile bk_rt: counted along, a division per unit costs more
+            // than the rest of this epilogue)
+            if (m[0] != m_before[0]) m_rt[0] = bk_rt;
+            if (m[1] != m_before[1]) m_rt[1] = bk_rt;
+            if (++bk_rt == RTP) { finish_image(bk_img); bk_img += groups; bk_rt = 0; }
         } else {
             m[0] = m[1] = INT_MIN;                           // there was no unit before the first
         }
@@ -564,7 +570,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     }
     {
         // the last unit's bookkeeping
-        const uint32_t u = nunits - 1, rt = u % RTP;
+        const uint32_t u = nunits - 1, rt = bk_rt;
         const int m_before[2] = {m[0], m[1]};
 #pragma unroll
         for (int j = 0; j < 16; ++j)
@@ -576,7 +582,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
             }
         if (m[0] != m_before[0]) m_rt[0] = rt;
         if (m[1] != m_before[1]) m_rt[1] = rt;
-        finish_image(grp + (u / RTP) * groups);              // units end with the last tile of an image
+        finish_image(bk_img);                                // units end with the last tile of an image
     }
 }
 
