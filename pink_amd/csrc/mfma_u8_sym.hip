@@ -399,24 +399,55 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     const uint32_t nrr = num_rot / 4;
     const uint32_t sym = col & 7;                          // same for both column tiles
 
-    // SOM-side fragments for the whole k range, and the row norms of this lane's two columns
-    v4i a[2][KS];
-    int na_l[2];
-    uint32_t n_l[2];
-#pragma unroll
-    for (int ct = 0; ct < 2; ++ct) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) a[ct][ks] = Pa[((size_t)(ct0 + ct) * KS + ks) * 64 + lane];
-        na_l[ct] = na[(ct0 + ct) * 32 + col];
-        n_l[ct] = ((ct0 + ct) * 32 + col) >> 3;
-    }
-    // pin the fragments to accumulation registers for the whole kernel: without this the compiler
-    // prefers to re-load them from memory for every row tile
-#pragma unroll
-    for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(a[ct][ks]));
     const bool sym_ok = (num_rot != 1 || (sym & 3) == 0) && (use_flip || (sym & 4) == 0);
+
+    // A wave whose two column tiles lie beyond the last neuron (the SOM's rows are padded to a whole
+    // number of blocks) has nothing to multiply: it only does its share of the staging, in step with
+    // the others through the block's barriers, and leaves the matrix pipe (and its power) alone.
+    // (A path of its own from the first instruction on, so that it shares no live values with the
+    // multiplying path, whose register allocation has no room to spare.)
+    if (__builtin_amdgcn_readfirstlane((int)(ct0 * 32 >= 8 * N))) {
+        const uint32_t images = grp < B ? (B - grp + groups - 1) / groups : 0;
+        const uint32_t units = images * RTP;
+        if (units == 0) return;
+        const v4i *from = Pb + (size_t)grp * RTP * UNIT_V + tid;
+        const size_t stride = (size_t)groups * RTP * UNIT_V;
+        uint32_t from_rt = 0, from_u = 0;
+        auto advance = [&]() {
+            ++from_u;
+            if (++from_rt == RTP) { from_rt = 0; from += stride - (size_t)(RTP - 1) * UNIT_V; }
+            else from += UNIT_V;
+        };
+        v4i held[PER_T];
+        int held_n;
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+        held_n = ((const int *)(from - tid + FRAG_V))[tid];
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) s_b[tid + 256 * i] = held[i];
+        s_n[0][tid] = held_n;
+        if (units > 1) advance();
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+        held_n = ((const int *)(from - tid + FRAG_V))[tid];
+        if (units > 2) advance();
+        __syncthreads();
+        uint32_t o_cur = 0, o_next = FRAG_V, o_free = 2 * FRAG_V;
+        for (uint32_t u = 0; u < units; ++u) {
+            v4i *dst = s_b + o_next + tid;
+#pragma unroll
+            for (int i = 0; i < PER_T; ++i) dst[256 * i] = held[i];
+            s_n[(u + 1) & 3][tid] = held_n;
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+            held_n = ((const int *)(from - tid + FRAG_V))[tid];
+            if (from_u + 1 < units) advance();
+            const uint32_t o = o_cur;
+            o_cur = o_next; o_next = o_free; o_free = o;
+        }
+        return;
+    }
 
     // The block's units: u -> image grp + (u / RTP) * groups, tile u % RTP.
     const uint32_t my_images = grp < B ? (B - grp + groups - 1) / groups : 0;
@@ -446,6 +477,25 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     stage_n = ((const int *)(src - tid + FRAG_V))[tid];
     if (nunits > 2) advance_src();
     __syncthreads();
+
+
+    // SOM-side fragments for the whole k range, and the row norms of this lane's two columns
+    v4i a[2][KS];
+    int na_l[2];
+    uint32_t n_l[2];
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) a[ct][ks] = Pa[((size_t)(ct0 + ct) * KS + ks) * 64 + lane];
+        na_l[ct] = na[(ct0 + ct) * 32 + col];
+        n_l[ct] = ((ct0 + ct) * 32 + col) >> 3;
+    }
+    // pin the fragments to accumulation registers for the whole kernel: without this the compiler
+    // prefers to re-load them from memory for every row tile
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(a[ct][ks]));
 
     // maximum over the 16 lanes that hold one neuron: the 8 symmetry lanes (two quad exchanges and
     // a mirror of the half row, all in the data-parallel path) and the other half-wave (v_permlane32_swap:
@@ -497,6 +547,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
 
     // LDS offsets (in vectors) of the buffers holding units u, u+1, u+2
     uint32_t off_cur = 0, off_next = FRAG_V, off_free = 2 * FRAG_V;
+
     v4i bf[4];
 #pragma unroll
     for (int ks = 0; ks < 3 && ks < KS; ++ks) bf[ks] = s_b[ks * 64 + lane];
