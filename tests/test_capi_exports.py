@@ -22,7 +22,8 @@ def test_library_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(L, name), "libpink_hip.so does not export " + name
     assert declared == set(capi.EXPORTS)
-    assert L.pink_hip_abi_version() == 2
+    version = int(re.search(r"#define\s+PINK_HIP_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "pink_hip.h")).read()).group(1))
+    assert L.pink_hip_abi_version() == version == 2
 
 
 @pytest.mark.parametrize("num_rot", [0, 3, 90, 6])
