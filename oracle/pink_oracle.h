@@ -22,6 +22,10 @@
  *     tests' known answers (290, {6,7,10,11}, 3-D best rotation, heatmap
  *     2.0/1.0/0.0, circular {0,.5,.2,.7}/{0,1,2,3}, update kernel vector)
  *     and by brute force in float64 / exact integers on small inputs.
+ *   - visiting order of the shuffled data iterator (libstdc++ 11's std::shuffle
+ *     over std::mt19937): compared with the reference's DataIteratorShuffled in
+ *     oracle/_ref, with orders taken from it (tests/golden/shuffle_orders.json)
+ *     and with the reference's own iterator test (seed 2, two entries).
  *   - integer (uint8/uint16) distance modes: the reference CPU path has none;
  *     the contract is the reference CPU functor evaluated in exact integers on
  *     arrays quantised as the reference's device conversion does
