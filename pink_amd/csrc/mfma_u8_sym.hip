@@ -562,13 +562,30 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
         v4i *dst = s_b + off_next + tid;
         const int m_before[2] = {m[0], m[1]};
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        auto book = [&](int t0, int t1) {
+        // The 32 (column, row) pairs of unit u-1 go through three steps -- sum of the two chains,
+        // shift and add of the norm entry, running maximum -- one pair behind the other: slot s does
+        // the sum of pair s, the shift-add of pair s-1 and the maximum of pair s-2, so that no step
+        // waits for the one before it in the same slot (a lone wave pays about 14 clocks per dependent
+        // vector instruction, and three of them in a row would hold up the next MFMA).
+        uint32_t pair_sum[2], pair_cand[2];
+        auto book = [&](int s0, int s1) {
 #pragma unroll
-            for (int t = t0; t < t1; ++t) {
-                const int ct = (t >> 2) & 1, j = 4 * (t >> 3) + (t & 3);
-                m[ct] = max(m[ct], (int)(((uint32_t)(acc_prev[ct][0][j] + acc_prev[ct][1][j]) << 5) + (uint32_t)cj_prev[j]));
+            for (int sl = s0; sl < s1; ++sl) {
+                if (sl >= 2 && sl < 34) {
+                    const int e = sl - 2, ct = (e >> 2) & 1;
+                    m[ct] = max(m[ct], (int)pair_cand[e & 1]);
+                }
+                if (sl >= 1 && sl < 33) {
+                    const int e = sl - 1, j = 4 * (e >> 3) + (e & 3);
+                    pair_cand[e & 1] = (pair_sum[e & 1] << 5) + (uint32_t)cj_prev[j];
+                }
+                if (sl < 32) {
+                    const int e = sl, ct = (e >> 2) & 1, j = 4 * (e >> 3) + (e & 3);
+                    pair_sum[e & 1] = (uint32_t)(acc_prev[ct][0][j] + acc_prev[ct][1][j]);
+                }
             }
-            asm volatile("" : "+v"(m[0]), "+v"(m[1]));      // pins the slice where it stands
+            // pins the slot where it stands
+            asm volatile("" : "+v"(m[0]), "+v"(m[1]), "+v"(pair_sum[0]), "+v"(pair_sum[1]), "+v"(pair_cand[0]), "+v"(pair_cand[1]));
         };
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -579,10 +596,10 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
             }
             bf[(ks + 3) & 3] = ks + 3 < KS ? cur[(ks + 3) * 64] : nxt[(ks + 3 - KS) * 64];
             acc[0][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[0][ks], ks > 1 ? acc[0][ks & 1] : zero, 0, 0, 0);
-            book((2 * ks) * 16 / KS, (2 * ks + 1) * 16 / KS);
+            book((2 * ks) * 17 / KS, (2 * ks + 1) * 17 / KS);
             __builtin_amdgcn_sched_barrier(0);
             acc[1][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[1][ks], ks > 1 ? acc[1][ks & 1] : zero, 0, 0, 0);
-            book((2 * ks + 1) * 16 / KS, (2 * ks + 2) * 16 / KS);
+            book((2 * ks + 1) * 17 / KS, (2 * ks + 2) * 17 / KS);
             // (past the last unit the staging moves data nobody reads: no branches in the k loop)
             if (ks >= W0 && ks < W0 + PER_T) dst[256 * (ks - W0)] = stage[ks - W0];
             if (ks == W0) s_n[(u + 1) & 3][tid] = stage_n;
