@@ -955,6 +955,8 @@ struct pink_hip_ctx {
     hipEvent_t st_ev[8] = {};              // per slot: the copy out of it has run
     uint32_t st_slot = 0;
     bool st_ring_busy = false;             // a call returned with copies out of the ring still queued
+    hipStream_t copy_stream = nullptr;     // host -> device copies of the next images while the kernels of the last run
+    hipEvent_t copy_ev[2] = {};
     uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
@@ -1335,6 +1337,8 @@ int free_all(pink_hip_ctx *ctx)
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
     for (hipEvent_t e : ctx->st_ev) if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : ctx->copy_ev) if (e) (void)hipEventDestroy(e);
+    if (ctx->copy_stream) (void)hipStreamDestroy(ctx->copy_stream);
     if (ctx->d_counts) (void)hipFree(ctx->d_counts);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
@@ -1899,6 +1903,42 @@ hipError_t stage_in(pink_hip_ctx *ctx, void *dev, const void *host, size_t bytes
     return hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream);
 }
 
+// `n` host images into the staging buffer and through `run(device images, first image, count)`,
+// in pieces of about 64 MB: the copy of a piece goes over a second stream while the kernels of the
+// piece before it run (also from pageable memory, where the copy call returns when the piece has
+// left the host buffer).  Small inputs take the pinned bounce buffer in one go.
+extern "C++" {
+template <typename Run>
+int staged_run(pink_hip_ctx *ctx, const float *host_images, uint32_t n, Run run)
+{
+    const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
+    if ((size_t)n * img_bytes <= kPinBytes) {
+        HIP_TRY(ctx, stage_in(ctx, ctx->st_img, host_images, n * img_bytes));
+        return run(ctx->st_img, 0u, n);
+    }
+    if (!ctx->copy_stream) {
+        HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->copy_stream, hipStreamNonBlocking));
+        for (hipEvent_t &e : ctx->copy_ev) HIP_TRY(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    }
+    // whatever still reads the staging buffer (queued per-image calls) finishes first
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    ctx->st_ring_busy = false;
+    uint32_t piece = (uint32_t)std::max<size_t>(1, ((size_t)64 << 20) / img_bytes);
+    if (piece > ctx->Bcap) piece -= piece % ctx->Bcap;     // whole launch groups
+    uint32_t turn = 0;
+    for (uint32_t first = 0; first < n; first += piece, turn ^= 1) {
+        const uint32_t count = std::min(piece, n - first);
+        float *dev = ctx->st_img + (size_t)first * ctx->isz;
+        HIP_TRY(ctx, hipMemcpyAsync(dev, host_images + (size_t)first * ctx->isz, count * img_bytes, hipMemcpyHostToDevice,
+                                    ctx->copy_stream));
+        HIP_TRY(ctx, hipEventRecord(ctx->copy_ev[turn], ctx->copy_stream));
+        HIP_TRY(ctx, hipStreamWaitEvent(ctx->stream, ctx->copy_ev[turn], 0));
+        TRY(run(dev, first, count));
+    }
+    return PINK_HIP_OK;
+}
+}  // extern "C++"
+
 int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out)
 {
     if (!ctx || (!host_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train: null argument");
@@ -1926,8 +1966,9 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
     TRY(ensure_staging(ctx, chunk));
     for (uint32_t done = 0; done < n_images; done += chunk) {
         const uint32_t n = std::min(chunk, n_images - done);
-        HIP_TRY(ctx, stage_in(ctx, ctx->st_img, host_images + (size_t)done * ctx->isz, n * img_bytes));
-        TRY(pink_hip_train_device(ctx, ctx->st_img, n, ctx->st_bmu));
+        TRY(staged_run(ctx, host_images + (size_t)done * ctx->isz, n, [&](const float *dev, uint32_t first, uint32_t count) {
+            return pink_hip_train_device(ctx, dev, count, ctx->st_bmu + first);
+        }));
         if (host_bmu_out) {
             const size_t out_bytes = n * sizeof(uint32_t);
             const bool small = out_bytes <= kPinBytes;
@@ -1969,8 +2010,9 @@ int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
     TRY(ensure_staging(ctx, chunk));
     for (uint32_t done = 0; done < n_images; done += chunk) {
         const uint32_t n = std::min(chunk, n_images - done);
-        HIP_TRY(ctx, stage_in(ctx, ctx->st_img, host_images + (size_t)done * ctx->isz, n * img_bytes));
-        TRY(pink_hip_map_device(ctx, ctx->st_img, n, ctx->st_heat, ctx->st_best));
+        TRY(staged_run(ctx, host_images + (size_t)done * ctx->isz, n, [&](const float *dev, uint32_t first, uint32_t count) {
+            return pink_hip_map_device(ctx, dev, count, ctx->st_heat + (size_t)first * ctx->N, ctx->st_best + (size_t)first * ctx->N);
+        }));
         const size_t heat_bytes = (size_t)n * ctx->N * sizeof(float);       // the best rotations take as many bytes
         const bool small = 2 * heat_bytes <= kPinBytes;
         char *pin_out = ctx->st_pin + kPinBytes;

@@ -329,6 +329,36 @@ def test_map_full_size_properties():
     assert np.array_equal(bits(heat3), bits(heat[:50]))
 
 
+def test_host_buffers_in_pieces_match_smaller_calls():
+    """Inputs beyond 64 MB go to the device piece by piece while the kernels of the piece before run:
+    the results are those of calls small enough to go in one piece."""
+    w = synthetic.WORKLOADS["cfg1"]
+    n = 9000                                                   # 147 MB of images: three pieces
+    imgs = synthetic.images(w, n)
+    say("pieces: map", n)
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(synthetic.initial_som(w))
+        heat, best = ctx.map(imgs)
+        parts = [ctx.map(imgs[i:i + 1500]) for i in range(0, n, 1500)]
+    assert np.array_equal(bits(heat), bits(np.concatenate([p[0] for p in parts])))
+    assert np.array_equal(best, np.concatenate([p[1] for p in parts]))
+    w = synthetic.WORKLOADS["cfg3"]
+    n = 1200                                                   # 144 MB of three-channel images: three pieces
+    imgs = synthetic.images(w, n)
+    tiny = dict(N=16, dims=[4, 4])
+    F = capi.make_update_factors(capi.CARTESIAN, tiny["dims"], capi.GAUSSIAN, 1.1, 0.2)
+    som0 = synthetic.mt19937_uniform(tiny["N"] * w.channels * 40 * 40, 7).reshape(tiny["N"], -1)
+    say("pieces: train", n)
+    results = []
+    for step in (n, 200):
+        with capi.Context(tiny["N"], w.channels, w.image_dim, 40, 8, True, 30, capi.QUADRATIC, capi.UINT8, F) as ctx:
+            ctx.set_som(som0)
+            bmu = np.concatenate([ctx.train(imgs[i:i + step]) for i in range(0, n, step)])
+            results.append((bmu, ctx.get_som(), ctx.update_counts()))
+    assert np.array_equal(results[0][0], results[1][0]) and np.array_equal(bits(results[0][1]), bits(results[1][1]))
+    assert np.array_equal(results[0][2], np.bincount(results[0][0], minlength=tiny["N"]))
+
+
 def test_empty_inputs_are_no_ops():
     w = synthetic.WORKLOADS["cfg4"]
     som = synthetic.initial_som(w)
