@@ -512,19 +512,27 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
 
     // Bookkeeping.  The unit's norm entry of row j of this lane is  cj = (15 - j) - 16 |b_row|^2, so
     //   cand = 32 acc_j + cj = 16 (|a|^2 - ssd_j) + (15 - j)       (|a|^2 = this column's norm)
-    // and the running signed maximum `m` of cand over rows and tiles is the minimum distance with
-    // the lowest row on ties; `m_rt` remembers the tile that set it (tiles ascend, a later tile
-    // must be strictly better).  16 ssd < 2^30 (checked on the host); rows beyond the last base
-    // rotation carry |b|^2 = 2^26 and never win.
-    int m[2] = {INT_MIN, INT_MIN};
+    // and the running signed maximum `m` of cand over the rows of a tile is the tile's minimum
+    // distance with the lowest row on ties.  Tiles ascend in rotation, so a later tile replaces the
+    // image's best so far (`best_m`, from tile `m_rt`) only with a strictly smaller distance: the
+    // comparison leaves the row bits out.  16 ssd < 2^30 (checked on the host); rows beyond the last
+    // base rotation carry |b|^2 = 2^26 and never win.
+    int m[2] = {INT_MIN, INT_MIN}, best_m[2] = {INT_MIN, INT_MIN};
     uint32_t m_rt[2] = {0, 0};
+    auto close_tile = [&](uint32_t rt) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+            if (rt == 0 || (m[ct] >> 4) > (best_m[ct] >> 4)) { best_m[ct] = m[ct]; m_rt[ct] = rt; }
+            m[ct] = INT_MIN;
+        }
+    };
     uint32_t bk_rt = 0, bk_img = grp;                      // tile and image of the unit whose bookkeeping ends next
     auto finish_image = [&](uint32_t b) {
         // lexicographic minimum of (distance, variant) over the neuron's 16 lanes in two passes
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-            const uint32_t j = 15u - ((uint32_t)m[ct] & 15u);
-            const int ssd = na_l[ct] - (m[ct] >> 4);
+            const uint32_t j = 15u - ((uint32_t)best_m[ct] & 15u);
+            const int ssd = na_l[ct] - (best_m[ct] >> 4);
             const uint32_t i = m_rt[ct] * 32 + 8 * (j >> 2) + 4 * half + (j & 3);
             const uint32_t k = (sym >> 2) * num_rot + (sym & 3) * nrr + i;
             const int sv = sym_ok ? -ssd : INT_MIN;
@@ -532,7 +540,6 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
             const int kmax = max16(sv == smax ? -(int)k : INT_MIN);
             if (half == 0 && sym == 0 && n_l[ct] < N)
                 key[(size_t)b * N + n_l[ct]] = ((unsigned long long)(uint32_t)(-smax) << 16) | (uint32_t)(-kmax);
-            m[ct] = INT_MIN;
         }
     };
     // this lane's 16 norm entries of unit u: rows 8g + 4*half .. +3, g = 0..3
@@ -560,7 +567,6 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     auto run_unit = [&](uint32_t u, v16i (&acc)[2][2], int (&cj)[16], const v16i (&acc_prev)[2][2], const int (&cj_prev)[16]) {
         const v4i *cur = s_b + off_cur + lane, *nxt = s_b + off_next + lane;
         v4i *dst = s_b + off_next + tid;
-        const int m_before[2] = {m[0], m[1]};
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         // The 32 (column, row) pairs of unit u-1 go through three steps -- sum of the two chains,
         // shift and add of the norm entry, running maximum -- one pair behind the other: slot s does
@@ -612,8 +618,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
         if (u > 0) {
             // (unit u - 1 = image bk_img, tile bk_rt: counted along, a division per unit costs more
             // than the rest of this epilogue)
-            if (m[0] != m_before[0]) m_rt[0] = bk_rt;
-            if (m[1] != m_before[1]) m_rt[1] = bk_rt;
+            close_tile(bk_rt);
             if (++bk_rt == RTP) { finish_image(bk_img); bk_img += groups; bk_rt = 0; }
         } else {
             m[0] = m[1] = INT_MIN;                           // there was no unit before the first
@@ -638,8 +643,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     }
     {
         // the last unit's bookkeeping
-        const uint32_t u = nunits - 1, rt = bk_rt;
-        const int m_before[2] = {m[0], m[1]};
+        const uint32_t u = nunits - 1;
 #pragma unroll
         for (int j = 0; j < 16; ++j)
 #pragma unroll
@@ -648,8 +652,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
                 const int cv = (u & 1) ? cj1[j] : cj0[j];
                 m[ct] = max(m[ct], (int)(((uint32_t)av << 5) + (uint32_t)cv));
             }
-        if (m[0] != m_before[0]) m_rt[0] = rt;
-        if (m[1] != m_before[1]) m_rt[1] = rt;
+        close_tile(bk_rt);
         finish_image(bk_img);                                // units end with the last tile of an image
     }
 }

@@ -191,6 +191,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         } else if constexpr (PACK >= 2) {
             // One work item = one 16-byte piece of one of the block's (up to 8) rows; the items of all
             // rows are dealt to the threads in one sequence, so the last round is the only partial one.
+            // The rows of the block are adjacent in the operand: nsym neighbouring lanes store 16 nsym
+            // consecutive bytes.
             // Four elements at a time: quantise (clamp, truncate), bytes gathered with v_perm, q - 128 (or
             // the two bytes of q - 32768 with the low one shifted by 128) = the bytes XOR 0x80, squares by
             // dot4: |256 h + l|^2 = 65536 h.h + 512 h.l + l.l.
@@ -205,8 +207,9 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                 return (uint32_t)v;
             };
             for (uint32_t item = threadIdx.x; item < nsym * pieces; item += blockDim.x) {
-                const uint32_t si = item / pieces, piece = item % pieces;
-                const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q, r = f * num_rot + q * nrr + i;
+                const uint32_t si = item % nsym, piece = item / nsym;   // neighbouring lanes: the adjacent rows of one piece
+                const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q;
+                const uint32_t r = i * nsym + si;             // operand row: the symmetries of a base rotation are adjacent
                 const uint4 *so4 = (const uint4 *)(pk.symoff + (size_t)sym * pk.Epad + piece * 16);
                 v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
                 int hh = 0, hl = 0, ll = 0;
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
             if (threadIdx.x < 8) {
                 const uint32_t f = threadIdx.x >> 2, q = threadIdx.x & 3;
                 if (f < nf && q < nq)
-                    pk.norm[(size_t)b * pk.rows_pad + f * num_rot + q * nrr + i] = (long long)s_norm[threadIdx.x];
+                    pk.norm[(size_t)b * pk.rows_pad + i * nsym + f * nq + q] = (long long)s_norm[threadIdx.x];
             }
         }
     } else {
@@ -975,6 +978,7 @@ struct pink_hip_ctx {
     bool gemm = false;
     uint32_t gKS = 0, Np = 0, Rp = 0, gslices = 1, gks_per = 0;   // k-slices (blocks per tile), k-steps per wave
     v4i *d_gPa = nullptr, *d_gPb = nullptr;
+    uint32_t *d_grow = nullptr, *d_gvariant = nullptr;   // variant index -> row of the variant operand, and back
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
 
@@ -1106,10 +1110,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
             hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(1024), 2 * ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr);
         else
             hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(1024), ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr);
         return launch_check(ctx, "k_pack_planes");
     }
     if (ctx->mfma_sym) {
@@ -1177,10 +1181,10 @@ int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
             hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(256), 2 * ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
-                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow);
         else
             hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(256), ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
-                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS);
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow);
         return launch_check(ctx, "k_pack_planes");
     }
     if (!is_int(ctx)) {
@@ -1261,6 +1265,7 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const long long *nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
     fin.nb = nb;
+    fin.variant = ctx->d_gvariant;
     if (slices == 1) {
         // a block sees the whole k range: it finishes its tile itself
         fin.key = key; fin.na = na; fin.na_other = na_other; fin.N = ctx->N; fin.R = ctx->R;
@@ -1271,7 +1276,7 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const uint32_t rows_per_chunk = 32;
     hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
                        dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, na, na_other, nb, key, ctx->N, ctx->Np, ctx->R,
-                       ctx->Rp, ctx->gslices, rows_per_chunk);
+                       ctx->Rp, ctx->gslices, rows_per_chunk, ctx->d_gvariant);
 }
 
 int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
@@ -1332,7 +1337,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
@@ -1584,6 +1589,23 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, &ctx->d_gPb, B * b_vec));
         TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)2 * ctx->Np));   // two halves, see na_cur
         TRY(dev_alloc(ctx, &ctx->d_gnb, B * ctx->Rp));
+        {
+            // rows of the variant operand: base rotation first, symmetry second
+            const uint32_t nq = c.num_rot == 1 ? 1u : 4u, nf = c.use_flip ? 2u : 1u, nsym = nq * nf;
+            const uint32_t nrr = std::max(c.num_rot / 4, 1u);
+            std::vector<uint32_t> row_of(ctx->R), variant_of(ctx->Rp, 0u);
+            for (uint32_t f = 0; f < nf; ++f)
+                for (uint32_t q = 0; q < nq; ++q)
+                    for (uint32_t i = 0; i < nrr; ++i) {
+                        const uint32_t k = f * c.num_rot + q * nrr + i, r = i * nsym + f * nq + q;
+                        row_of[k] = r;
+                        variant_of[r] = k;
+                    }
+            TRY(dev_alloc(ctx, &ctx->d_grow, row_of.size()));
+            TRY(dev_alloc(ctx, &ctx->d_gvariant, variant_of.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_grow, row_of.data(), row_of.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_gvariant, variant_of.data(), variant_of.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        }
         TRY(dev_alloc(ctx, &ctx->d_dot, dot_n));
         // rows beyond N / R and elements beyond the region are never written: they must read as zero
         HIP_TRY(ctx, hipMemset(ctx->d_gPa, 0, a_vec * sizeof(v4i)));

@@ -220,6 +220,7 @@ SYM_SHAPES = [
     (12, 1, 16, 12, 1, True, 12, capi.QUADRATIC, 4),       # flip only
     (25, 1, 40, 29, 16, True, 21, capi.CIRCULAR, 7),       # circular region, odd diameter
     (1, 1, 28, 28, 360, True, 28, capi.QUADRATIC, 1),      # a single neuron, a single image
+    (3, 2, 6, 7, 360, True, 1, capi.QUADRATIC, 3),         # a one-pixel region: equal distances all over, the first variant wins
 ]
 
 
@@ -250,6 +251,32 @@ def test_map_uint8_kernels_over_shapes(N, C_, I, D, nrot, flip, ed, shape_, n):
         assert np.array_equal(bits(heat_again), bits(oheat[:1])) and np.array_equal(best_again, obest[:1]), choice
     say("   kernels that ran:", ran)
     assert capi.KERNEL_MFMA_GEMM in ran and capi.KERNEL_MFMA_SYM in ran
+
+
+@pytest.mark.parametrize("ed_type", [capi.FLOAT, capi.UINT8, capi.UINT16])
+def test_equal_distances_go_to_the_first_variant(ed_type):
+    """A constant image has 720 identical quantised variants: every kernel must report variant 0 for every neuron
+    (strict `<` over ascending variants, generate_euclidean_distance_matrix.h:43-50), also where the
+    equal distances sit in different tiles of rotations."""
+    N, C_, I, D, nrot, flip, ed = 9, 1, 32, 22, 360, True, 16
+    rng = np.random.default_rng(17)
+    som = rng.random((N, D * D), dtype=np.float32)
+    imgs = np.full((2, C_, I, I), 0.5, np.float32)
+    imgs[1, 0, 8:24, 8:24] = 0.25                     # constant inside every rotated region, not outside
+    s = O.shape(N, C_, I, D, nrot, flip, ed, O.QUADRATIC, ed_type)
+    oheat, obest = O.map_images(s, som, imgs)
+    if ed_type != capi.FLOAT:                          # (in float32 the interpolation weights do not sum to exactly 1)
+        assert (obest[0] == 0).all()
+    choices = [capi.KERNEL_AUTO] if ed_type == capi.FLOAT else [capi.KERNEL_AUTO, capi.KERNEL_VALU, capi.KERNEL_MFMA_GEMM]
+    if ed_type == capi.UINT8:
+        choices += [capi.KERNEL_MFMA, capi.KERNEL_MFMA_SYM]
+    for choice in choices:
+        say("ties", ed_type, choice)
+        with capi.Context(N, C_, I, D, nrot, flip, ed, capi.QUADRATIC, ed_type, kernel_choice=choice) as ctx:
+            ctx.set_som(som)
+            heat, best = ctx.map(imgs)
+        assert np.array_equal(best, obest), choice
+        assert np.array_equal(bits(heat), bits(oheat)), choice
 
 
 FUSED_TRAIN_SHAPES = [
