@@ -283,7 +283,8 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
         uint32_t live[4];                                 // byte masks of the positions inside the union
 #pragma unroll
         for (int w4 = 0; w4 < 4; ++w4) {
-            const int inside = (int)Ku - (int)(k0 + 4 * w4);
+            // (rows beyond the last base rotation are all zero: their products must not count)
+            const int inside = i < nrr_eff ? (int)Ku - (int)(k0 + 4 * w4) : 0;
             live[w4] = inside >= 4 ? 0xffffffffu : inside <= 0 ? 0u : (1u << (8 * inside)) - 1u;
         }
         if (i < nrr_eff) {
@@ -359,7 +360,9 @@ __global__ __launch_bounds__(512) void k_rotpack_sym_u8(const float *__restrict_
         // index the distance kernel's lanes hold this row in (see there).  Rows beyond the last base
         // rotation get a norm no real distance reaches: they never win the argmin.
         const uint32_t s = threadIdx.x >> 5, g = threadIdx.x & 31;
-        const int norm = rt * 32 + g < nrr_eff ? (all_sym ? s_nb[gi][g][0] : s_nb[gi][g][s]) : (1 << 26);
+        // (16 times the stand-in must stay inside int32 and below 16 (ssd - |a|^2) of any real row:
+        // real rows reach 16 * 9.96e7 at 2048 elements)
+        const int norm = rt * 32 + g < nrr_eff ? (all_sym ? s_nb[gi][g][0] : s_nb[gi][g][s]) : (KS > 32 ? (1 << 27) - 1 : (1 << 26));
         const int j = 4 * (g >> 3) + (g & 3);
         int *entries = (int *)(Pb + ((size_t)(b0 + gi) * RTP + rt) * UNIT_V + KS * 64);
         entries[s * 32 + g] = (15 - j) - 16 * norm;
@@ -657,6 +660,216 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     }
 }
 
+// The same for unions of up to 2048 elements (KS = 40 .. 64 k-steps): a wave's accumulation registers
+// hold ONE column tile over the whole k range (4 neurons x 8 symmetries), a block 4 tiles; a unit is
+// up to 64 KiB, so two LDS buffers take turns and a unit has two barriers: the first, early in
+// the k loop, says that every wave has left the previous unit (whose buffer then receives unit u+1 from
+// the staging registers), the second that those stores have landed (the fragment reads run on into the
+// next buffer at the end of the k loop).  One MFMA per k-step and fragment read, two chains (even /
+// odd k-steps); bookkeeping, half-wave exchange and keys as above.
+template <int KS>
+__global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8_wide(const v4i *__restrict__ Pa, const int *__restrict__ na,
+                                                                  const v4i *__restrict__ Pb,
+                                                                  unsigned long long *__restrict__ key, uint32_t N,
+                                                                  uint32_t B, uint32_t num_rot, uint32_t use_flip,
+                                                                  uint32_t RTP, uint32_t groups)
+{
+    constexpr int FRAG_V = KS * 64;
+    constexpr int UNIT_V = FRAG_V + 64;
+    constexpr int PER_T = KS / 4;
+    constexpr int W0 = 2, H2 = W0 + PER_T + 2, L0 = H2;    // first barrier and stores / second barrier / loads
+    static_assert(KS % 8 == 0 && L0 + PER_T <= KS - 3, "k loop too short for the staging schedule");
+    extern __shared__ v4i s_b[];                           // 2 x FRAG_V
+    __shared__ int s_n[4][256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t col = lane & 31, half = lane >> 5;
+    const uint32_t slice = blockIdx.x / groups, grp = blockIdx.x % groups;
+    const uint32_t ct = slice * 4 + wave;                  // this wave's column tile
+    const uint32_t nrr = num_rot / 4;
+    const uint32_t sym = col & 7;
+    const bool sym_ok = (num_rot != 1 || (sym & 3) == 0) && (use_flip || (sym & 4) == 0);
+
+    // a wave whose column tile lies beyond the last neuron only takes part in the staging (a path of
+    // its own from here on, sharing no live values with the multiplying path)
+    if (__builtin_amdgcn_readfirstlane((int)(ct * 32 >= 8 * N))) {
+        const uint32_t images = grp < B ? (B - grp + groups - 1) / groups : 0;
+        const uint32_t units = images * RTP;
+        if (units == 0) return;
+        const v4i *from = Pb + (size_t)grp * RTP * UNIT_V + tid;
+        const size_t stride = (size_t)groups * RTP * UNIT_V;
+        uint32_t from_rt = 0, from_u = 0;
+        auto advance = [&]() {
+            ++from_u;
+            if (++from_rt == RTP) { from_rt = 0; from += stride - (size_t)(RTP - 1) * UNIT_V; }
+            else from += UNIT_V;
+        };
+        v4i held[PER_T];
+        int held_n;
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+        held_n = ((const int *)(from - tid + FRAG_V))[tid];
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) s_b[tid + 256 * i] = held[i];
+        s_n[0][tid] = held_n;
+        if (units > 1) advance();
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+        held_n = ((const int *)(from - tid + FRAG_V))[tid];
+        if (units > 2) advance();
+        __syncthreads();
+        uint32_t o_cur = 0, o_next = FRAG_V;
+        for (uint32_t u = 0; u < units; ++u) {
+            asm volatile("s_barrier" ::: "memory");
+            v4i *dst = s_b + o_next + tid;
+#pragma unroll
+            for (int i = 0; i < PER_T; ++i) dst[256 * i] = held[i];
+            s_n[(u + 1) & 3][tid] = held_n;
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < PER_T; ++i) held[i] = from[256 * i];
+            held_n = ((const int *)(from - tid + FRAG_V))[tid];
+            if (from_u + 1 < units) advance();
+            const uint32_t o = o_cur;
+            o_cur = o_next; o_next = o;
+        }
+        return;
+    }
+
+    const uint32_t my_images = grp < B ? (B - grp + groups - 1) / groups : 0;
+    const uint32_t nunits = my_images * RTP;
+    if (nunits == 0) return;
+    const v4i *src = Pb + (size_t)grp * RTP * UNIT_V + tid;
+    const size_t image_stride = (size_t)groups * RTP * UNIT_V;
+    uint32_t src_rt = 0, src_u = 0;
+    auto advance_src = [&]() {
+        ++src_u;
+        if (++src_rt == RTP) { src_rt = 0; src += image_stride - (size_t)(RTP - 1) * UNIT_V; }
+        else src += UNIT_V;
+    };
+    v4i stage[PER_T];
+    int stage_n;
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) stage[i] = src[256 * i];
+    stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) s_b[tid + 256 * i] = stage[i];
+    s_n[0][tid] = stage_n;
+    if (nunits > 1) advance_src();
+#pragma unroll
+    for (int i = 0; i < PER_T; ++i) stage[i] = src[256 * i];
+    stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+    if (nunits > 2) advance_src();
+    __syncthreads();
+    uint32_t off_cur = 0, off_next = FRAG_V;
+
+
+    v4i a[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a[ks] = Pa[((size_t)ct * KS + ks) * 64 + lane];
+    const int na_l = na[ct * 32 + col];
+    const uint32_t n_l = (ct * 32 + col) >> 3;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(a[ks]));
+
+    auto max16 = [&](int v) -> int {
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));
+        v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));
+        const auto halves = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+        return max((int)halves[0], (int)halves[1]);
+    };
+    int m = INT_MIN, best_m = INT_MIN;
+    uint32_t m_rt = 0;
+    uint32_t bk_rt = 0, bk_img = grp;
+    auto close_tile = [&](uint32_t rt) {
+        if (rt == 0 || (m >> 4) > (best_m >> 4)) { best_m = m; m_rt = rt; }
+        m = INT_MIN;
+    };
+    auto finish_image = [&](uint32_t b) {
+        const uint32_t j = 15u - ((uint32_t)best_m & 15u);
+        const int ssd = na_l - (best_m >> 4);
+        const uint32_t i = m_rt * 32 + 8 * (j >> 2) + 4 * half + (j & 3);
+        const uint32_t k = (sym >> 2) * num_rot + (sym & 3) * nrr + i;
+        const int sv = sym_ok ? -ssd : INT_MIN;
+        const int smax = max16(sv);
+        const int kmax = max16(sv == smax ? -(int)k : INT_MIN);
+        if (half == 0 && sym == 0 && n_l < N)
+            key[(size_t)b * N + n_l] = ((unsigned long long)(uint32_t)(-smax) << 16) | (uint32_t)(-kmax);
+    };
+    auto read_cj = [&](uint32_t u, int (&cj)[16]) {
+        const v4i *nbt = (const v4i *)(&s_n[u & 3][sym * 32 + 4 * half]);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const v4i t = nbt[2 * g];
+            cj[4 * g + 0] = t[0]; cj[4 * g + 1] = t[1]; cj[4 * g + 2] = t[2]; cj[4 * g + 3] = t[3];
+        }
+    };
+
+    v4i bf[4];
+#pragma unroll
+    for (int ks = 0; ks < 3; ++ks) bf[ks] = s_b[ks * 64 + lane];
+
+    auto run_unit = [&](uint32_t u, v16i (&acc)[2], int (&cj)[16], const v16i (&acc_prev)[2], const int (&cj_prev)[16]) {
+        const v4i *cur = s_b + off_cur + lane, *nxt = s_b + off_next + lane;
+        v4i *dst = s_b + off_next + tid;
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        // the 16 rows of unit u-1 in three steps, one row behind the other (see the kernel above)
+        uint32_t pair_sum[2], pair_cand[2];
+        auto book = [&](int s0, int s1) {
+#pragma unroll
+            for (int sl = s0; sl < s1; ++sl) {
+                if (sl >= 2 && sl < 18) m = max(m, (int)pair_cand[sl & 1]);
+                if (sl >= 1 && sl < 17) pair_cand[(sl - 1) & 1] = (pair_sum[(sl - 1) & 1] << 5) + (uint32_t)cj_prev[sl - 1];
+                if (sl < 16) pair_sum[sl & 1] = (uint32_t)(acc_prev[0][sl] + acc_prev[1][sl]);
+            }
+            asm volatile("" : "+v"(m), "+v"(pair_sum[0]), "+v"(pair_sum[1]), "+v"(pair_cand[0]), "+v"(pair_cand[1]));
+        };
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks == W0) asm volatile("s_barrier" ::: "memory");          // every wave has left unit u-1
+            if (ks == H2) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // unit u+1 is in LDS
+            bf[(ks + 3) & 3] = ks + 3 < KS ? cur[(ks + 3) * 64] : nxt[(ks + 3 - KS) * 64];
+            acc[ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[ks], ks > 1 ? acc[ks & 1] : zero, 0, 0, 0);
+            book(ks * 18 / KS, (ks + 1) * 18 / KS);
+            if (ks >= W0 && ks < W0 + PER_T) dst[256 * (ks - W0)] = stage[ks - W0];
+            if (ks == W0) s_n[(u + 1) & 3][tid] = stage_n;
+            if (ks >= L0 && ks < L0 + PER_T) stage[ks - L0] = src[256 * (ks - L0)];
+            if (ks == L0) stage_n = ((const int *)(src - tid + FRAG_V))[tid];
+            if (ks == KS - 2) read_cj(u, cj);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (src_u + 1 < nunits) advance_src();
+        if (u > 0) {
+            close_tile(bk_rt);
+            if (++bk_rt == RTP) { finish_image(bk_img); bk_img += groups; bk_rt = 0; }
+        } else {
+            m = INT_MIN;
+        }
+        const uint32_t o = off_cur;
+        off_cur = off_next; off_next = o;
+    };
+
+    v16i acc0[2], acc1[2];
+    int cj0[16], cj1[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) { acc1[0][j] = acc1[1][j] = 0; cj1[j] = 0; }
+    for (uint32_t u = 0; u < nunits; u += 2) {
+        run_unit(u, acc0, cj0, acc1, cj1);
+        if (u + 1 < nunits) run_unit(u + 1, acc1, cj1, acc0, cj0);
+    }
+    {
+        const uint32_t u = nunits - 1;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int av = (u & 1) ? acc1[0][j] + acc1[1][j] : acc0[0][j] + acc0[1][j];
+            const int cv = (u & 1) ? cj1[j] : cj0[j];
+            m = max(m, (int)(((uint32_t)av << 5) + (uint32_t)cv));
+        }
+        close_tile(bk_rt);
+        finish_image(bk_img);
+    }
+}
+
 template <int KS>
 hipError_t launch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool configure_only)
 {
@@ -668,6 +881,17 @@ hipError_t launch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool con
     return hipGetLastError();
 }
 
+template <int KS>
+hipError_t launch_dist_wide(hipStream_t stream, const pink_sym::DistArgs &g, bool configure_only)
+{
+    const int lds = 2 * KS * 64 * 16;
+    if (configure_only)
+        return hipFuncSetAttribute((const void *)k_dist_mfma_sym_u8_wide<KS>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipLaunchKernelGGL((k_dist_mfma_sym_u8_wide<KS>), dim3(g.slices * g.groups), dim3(256), lds, stream, (const v4i *)g.Pa,
+                       g.na, (const v4i *)g.Pb, g.key, g.N, g.B, g.num_rot, g.use_flip, g.RTP, g.groups);
+    return hipGetLastError();
+}
+
 hipError_t dispatch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool configure_only)
 {
     switch (g.KS) {
@@ -675,6 +899,10 @@ hipError_t dispatch_dist(hipStream_t stream, const pink_sym::DistArgs &g, bool c
     case 16: return launch_dist<16>(stream, g, configure_only);
     case 24: return launch_dist<24>(stream, g, configure_only);
     case 32: return launch_dist<32>(stream, g, configure_only);
+    case 40: return launch_dist_wide<40>(stream, g, configure_only);
+    case 48: return launch_dist_wide<48>(stream, g, configure_only);
+    case 56: return launch_dist_wide<56>(stream, g, configure_only);
+    case 64: return launch_dist_wide<64>(stream, g, configure_only);
     default: return hipErrorInvalidValue;
     }
 }

@@ -970,7 +970,7 @@ struct pink_hip_ctx {
     uint32_t *d_need = nullptr;
     // uint8 mapping with the symmetries on the SOM side
     bool mfma_sym = false;
-    uint32_t Ku = 0, KSs = 0, RTP = 0, slices = 0, groups = 1, all_sym = 0;
+    uint32_t Ku = 0, KSs = 0, RTP = 0, slices = 0, groups = 1, all_sym = 0, sym_tiles = 8;
     uint32_t *d_upos = nullptr, *d_aoff = nullptr;
     unsigned char *d_kmask = nullptr;
 
@@ -1118,7 +1118,7 @@ int run_pack_som(pink_hip_ctx *ctx)
     }
     if (ctx->mfma_sym) {
         HIP_TRY(ctx, pink_sym::pack_som(ctx->stream, ctx->d_som, ctx->d_aoff, ctx->d_Pa, ctx->d_na, ctx->N, ctx->S, ctx->KSs,
-                                        ctx->slices * 8 * 32));
+                                        ctx->slices * ctx->sym_tiles * 32));
         return PINK_HIP_OK;
     }
     if (ctx->mfma) {
@@ -1436,10 +1436,11 @@ int init_ctx(pink_hip_ctx *ctx)
             }
         ctx->Ku = (uint32_t)upos.size();
         const uint32_t ks_need = (ctx->Ku + 31) / 32;
-        ctx->KSs = ks_need <= 8 ? 8 : ks_need <= 16 ? 16 : ks_need <= 24 ? 24 : 32;
+        ctx->KSs = (ks_need + 7) / 8 * 8;                  // 8 .. 32: two column tiles per wave; 40 .. 64: one
+        ctx->sym_tiles = ctx->KSs <= 32 ? 8 : 4;           // column tiles per block (4 waves)
         ctx->RTP = (ctx->nrr_eff + 31) / 32;
         const uint32_t col_tiles = (8 * ctx->N + 31) / 32;
-        ctx->slices = (col_tiles + 7) / 8;                 // 4 waves x 2 column tiles per block
+        ctx->slices = (col_tiles + ctx->sym_tiles - 1) / ctx->sym_tiles;
         ctx->groups = std::max(1u, (uint32_t)ctx->num_cu / ctx->slices);
         // a region element must not repeat (the multi-channel circular rule repeats channel 0)
         bool distinct = true;
@@ -1448,10 +1449,10 @@ int init_ctx(pink_hip_ctx *ctx)
             for (uint32_t e = 0; e < ctx->E; ++e) { if (seen[region[e]]) distinct = false; seen[region[e]] = 1; }
         }
         const size_t lds_img = pink_sym::lds_image_bytes(ctx->C, ctx->I);
-        const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 32 && ctx->RTP <= 3 &&
+        const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 64 && ctx->RTP <= 3 &&
                               lds_img <= 150 * 1024 && D < 4096 && ctx->C < 256;
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM && !fits_sym)
-            return fail(ctx, PINK_HIP_EINVAL, "the symmetric MFMA distance kernel needs a uint8 mapper, at most 1024 "
+            return fail(ctx, PINK_HIP_EINVAL, "the symmetric MFMA distance kernel needs a uint8 mapper, at most 2048 "
                                               "region elements (union over the symmetries) and at most 384 rotations");
         ctx->mfma_sym = fits_sym && (c.kernel_choice == PINK_HIP_KERNEL_AUTO || c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM);
         if (ctx->mfma_sym) {
@@ -1578,8 +1579,8 @@ int init_ctx(pink_hip_ctx *ctx)
     TRY(dev_alloc(ctx, &ctx->d_rot, ((ctx->mfma || ctx->mfma_sym) ? 1 : B) * ctx->R * ctx->S));
     TRY(dev_alloc(ctx, &ctx->d_key, B * ctx->N));
     if (ctx->mfma_sym) {
-        TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->slices * 8 * ctx->KSs * 1024));
-        TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->slices * 8 * 32));
+        TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->slices * ctx->sym_tiles * ctx->KSs * 1024));
+        TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->slices * ctx->sym_tiles * 32));
         TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RTP * pink_sym::unit_bytes(ctx->KSs)));
     } else if (ctx->gemm) {
         const size_t planes = c.ed_type == PINK_HIP_UINT16 ? 2 : 1;

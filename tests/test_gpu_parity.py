@@ -221,6 +221,10 @@ SYM_SHAPES = [
     (25, 1, 40, 29, 16, True, 21, capi.CIRCULAR, 7),       # circular region, odd diameter
     (1, 1, 28, 28, 360, True, 28, capi.QUADRATIC, 1),      # a single neuron, a single image
     (3, 2, 6, 7, 360, True, 1, capi.QUADRATIC, 3),         # a one-pixel region: equal distances all over, the first variant wins
+    (37, 1, 64, 91, 360, True, 45, capi.QUADRATIC, 9),     # 2025 elements: the wide form (64 k-steps, one column tile per wave)
+    (130, 1, 64, 64, 360, True, 44, capi.CIRCULAR, 2),     # wide form, 48 k-steps, nine slices
+    (9, 1, 52, 42, 360, True, 38, capi.QUADRATIC, 40),     # wide form, several images per group
+    (20, 2, 40, 30, 360, False, 30, capi.QUADRATIC, 4),    # wide form, two channels, no flip
 ]
 
 
@@ -277,6 +281,37 @@ def test_equal_distances_go_to_the_first_variant(ed_type):
             heat, best = ctx.map(imgs)
         assert np.array_equal(best, obest), choice
         assert np.array_equal(bits(heat), bits(oheat)), choice
+
+
+@pytest.mark.parametrize("ed", [32, 45])
+def test_largest_distances_do_not_lose_to_padding(ed):
+    """Neurons of zeros against images of ones (and the reverse) give the largest distances a region
+    allows: they must still beat the padded rows and columns of every integer kernel (ed = 45, 2025
+    elements, takes the wide form of the symmetric kernel)."""
+    N, C_, I, D, nrot, flip = 6, 1, 64, (44 if ed == 32 else 91), 360, True
+    rng = np.random.default_rng(ed)
+    som = rng.random((N, D * D), dtype=np.float32)
+    som[0] = 0.0
+    som[1] = 1.0
+    imgs = rng.random((4, C_, I, I), dtype=np.float32)
+    imgs[0] = 1.0
+    imgs[1] = 0.0
+    for ed_type in (capi.UINT8, capi.UINT16):
+        s = O.shape(N, C_, I, D, nrot, flip, ed, O.QUADRATIC, ed_type)
+        oheat, obest = O.map_images(s, som, imgs)
+        choices = [capi.KERNEL_AUTO, capi.KERNEL_MFMA_GEMM] + ([capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA] if ed_type == capi.UINT8 else [])
+        for choice in choices:
+            say("extremes", ed, ed_type, choice)
+            try:
+                ctx = capi.Context(N, C_, I, D, nrot, flip, ed, capi.QUADRATIC, ed_type, kernel_choice=choice)
+            except capi.PinkError:
+                assert choice == capi.KERNEL_MFMA
+                continue
+            with ctx:
+                ctx.set_som(som)
+                heat, best = ctx.map(imgs)
+            assert np.array_equal(bits(heat), bits(oheat)), (ed_type, choice)
+            assert np.array_equal(best, obest), (ed_type, choice)
 
 
 FUSED_TRAIN_SHAPES = [
