@@ -137,7 +137,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
-                                                uint32_t use_flip, uint32_t use_lds, uint32_t Dp, PackArgs pk)
+                                                uint32_t use_flip, uint32_t use_lds, uint32_t Dp, PackArgs pk,
+                                                uint32_t store_variants)
 {
     // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
     // stride keeps those reads in different banks (a stride of 64 would put all of them into one)
@@ -160,7 +161,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x)
             s_base[(p / D) * Dp + p % D] = base_pixel(img, I, D, i, cs, sn, p / D, p % D);
         __syncthreads();
-        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
+        // (a mapper whose distance operand is packed below never reads the variants themselves)
+        for (uint32_t p = threadIdx.x; p < (store_variants ? DD : 0u); p += blockDim.x) {
             const uint32_t x = p / D, y = p % D;
             for (uint32_t f = 0; f < nf; ++f) {
                 const uint32_t xs = f ? D - 1 - x : x;
@@ -1137,7 +1139,7 @@ int run_pack_som(pink_hip_ctx *ctx)
     return launch_check(ctx, "k_pack_som");
 }
 
-int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
+int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, bool store_variants = true)
 {
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
@@ -1163,7 +1165,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
 #define LAUNCH_ROTATE(P_)                                                                                          \
     hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
-                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk)
+                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store_variants ? 1u : 0u)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
     case 2: LAUNCH_ROTATE(2); break;
@@ -1744,7 +1746,8 @@ int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
         TRY(run_dist_mfma(ctx, B));
         return PINK_HIP_OK;
     }
-    TRY(run_rotate(ctx, dev_images, B));
+    // the variants themselves are only read by the update kernel and by a separate packing kernel
+    TRY(run_rotate(ctx, dev_images, B, ctx->trainer || !ctx->fused_pack));
     TRY(run_pack_rot(ctx, B));
     TRY(run_dist(ctx, 0, B));
     return PINK_HIP_OK;
