@@ -138,7 +138,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
                                                 uint32_t use_flip, uint32_t use_lds, uint32_t Dp, PackArgs pk,
-                                                uint32_t store_variants)
+                                                uint32_t store_variants, uint32_t lo, uint32_t hi)
 {
     // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
     // stride keeps those reads in different banks (a stride of 64 would put all of them into one)
@@ -158,8 +158,13 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     if (PACK >= 2 && threadIdx.x < 8) s_norm[threadIdx.x] = 0;
 
     if (use_lds) {
-        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x)
-            s_base[(p / D) * Dp + p % D] = base_pixel(img, I, D, i, cs, sn, p / D, p % D);
+        // rows and columns [lo, hi) of the base rotation: all of it, or, when only the packed operand is
+        // wanted, the square that the region reaches under the eight symmetries
+        const uint32_t side = hi - lo;
+        for (uint32_t p = threadIdx.x; p < side * side; p += blockDim.x) {
+            const uint32_t x = lo + p / side, y = lo + p % side;
+            s_base[x * Dp + y] = base_pixel(img, I, D, i, cs, sn, x, y);
+        }
         __syncthreads();
         // (a mapper whose distance operand is packed below never reads the variants themselves)
         for (uint32_t p = threadIdx.x; p < (store_variants ? DD : 0u); p += blockDim.x) {
@@ -926,6 +931,7 @@ struct pink_hip_ctx {
     uint32_t isz = 0;          // floats per image
     uint32_t Bcap = 1;         // images per launch group
     uint32_t Dp = 0;           // row stride of the rotation kernel's LDS tile
+    uint32_t base_lo = 0, base_hi = 0;   // rows and columns of a base rotation that the packed region reads
     uint32_t shift = 32;       // key = value << shift | rotation
     uint32_t factor = 1;       // 255 / 65535 in the integer modes
     bool trainer = false;
@@ -1165,7 +1171,8 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, bool stor
 #define LAUNCH_ROTATE(P_)                                                                                          \
     hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
-                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store_variants ? 1u : 0u)
+                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store_variants ? 1u : 0u,                   \
+                       store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
     case 2: LAUNCH_ROTATE(2); break;
@@ -1632,6 +1639,7 @@ int init_ctx(pink_hip_ctx *ctx)
     if (ctx->fused_pack) {
         const uint32_t D = ctx->D, DD = D * D;
         std::vector<uint32_t> symoff((size_t)8 * ctx->Epad, 0u);
+        ctx->base_lo = D; ctx->base_hi = 0;
         for (uint32_t sym = 0; sym < 8; ++sym) {
             const uint32_t f = sym >> 2, q = sym & 3;
             for (uint32_t e = 0; e < ctx->E; ++e) {
@@ -1647,8 +1655,11 @@ int init_ctx(pink_hip_ctx *ctx)
                 default: a = y; bb = D - 1 - xs; break;
                 }
                 symoff[(size_t)sym * ctx->Epad + e] = (ch << 24) | (a * ctx->Dp + bb);     // LDS rows of Dp floats
+                ctx->base_lo = std::min({ctx->base_lo, a, bb});
+                ctx->base_hi = std::max({ctx->base_hi, a + 1, bb + 1});
             }
         }
+        if (ctx->base_hi <= ctx->base_lo) ctx->base_lo = ctx->base_hi = 0;       // empty region
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
         HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, symoff.data(), symoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
     }
