@@ -1558,6 +1558,16 @@ int init_ctx(pink_hip_ctx *ctx)
         }
     }
 
+    ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
+    ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= 64 * 1024;
+    // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
+    // integer contexts, whenever the kernel keeps its base rotation in LDS.
+    ctx->fused_pack = ctx->use_lds && !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && ctx->D <= 4096 &&
+                      (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
+    // Float variants of a whole launch group: for the update kernel and for a separate packing kernel.
+    // The other contexts keep room for one image (pink_hip_rotate).
+    const bool group_variants = ctx->trainer || !(ctx->mfma || ctx->mfma_sym || ctx->fused_pack);
+
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
     size_t per_image = ((size_t)ctx->R * ctx->S + (size_t)ctx->Epad * ctx->Rpad) * 4 + (size_t)ctx->N * 24;
     if (ctx->mfma) per_image = (size_t)ctx->RT * ctx->KS * 1024 + (size_t)ctx->RT * 128 + (size_t)ctx->N * 24;
@@ -1565,6 +1575,7 @@ int init_ctx(pink_hip_ctx *ctx)
         per_image = (size_t)ctx->R * ctx->S * 4 + (size_t)(c.ed_type == PINK_HIP_UINT16 ? 2 : 1) * (ctx->Rp / 32) * ctx->gKS * 1024 +
                     (size_t)ctx->Rp * 8 + (size_t)ctx->N * 24;
     if (ctx->mfma_sym) per_image = (size_t)ctx->RTP * pink_sym::unit_bytes(ctx->KSs) + (size_t)ctx->N * 24;
+    else if (!ctx->mfma && !group_variants) per_image -= (size_t)ctx->R * ctx->S * 4;
     if (ctx->trainer) {
         // images whose variants are prepared ahead of the sequential distance/update chain
         size_t b = c.max_batch ? c.max_batch : 64;
@@ -1575,17 +1586,20 @@ int init_ctx(pink_hip_ctx *ctx)
         size_t b = c.max_batch ? c.max_batch : ((ctx->mfma || ctx->mfma_sym) ? 2048 : 256);
         const size_t budget = (size_t)4 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
+        if (ctx->gemm && !c.max_batch) {
+            // the GEMM reads a group's variant operand right after the rotation kernel wrote it: a group whose
+            // operand stays within the 256 MB last-level cache maps faster than a larger one (measured: the
+            // optimum is the largest power of two with at most ~190 MB, 128 images at 2048 uint8 elements)
+            const size_t operand = (size_t)(c.ed_type == PINK_HIP_UINT16 ? 2 : 1) * (ctx->Rp / 32) * ctx->gKS * 1024;
+            while (b > 16 && b * operand > ((size_t)192 << 20)) b >>= 1;
+        }
         ctx->Bcap = (uint32_t)b;
     }
     const size_t B = ctx->Bcap;
-    ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
-    ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= 64 * 1024;
 
     TRY(dev_alloc(ctx, &ctx->d_som, (size_t)ctx->N * ctx->S));
     HIP_TRY(ctx, hipMemset(ctx->d_som, 0, (size_t)ctx->N * ctx->S * sizeof(float)));
-    // The float variants are only materialised per launch group on the vector-ALU path; the
-    // matrix-core path keeps room for one image (pink_hip_rotate).
-    TRY(dev_alloc(ctx, &ctx->d_rot, ((ctx->mfma || ctx->mfma_sym) ? 1 : B) * ctx->R * ctx->S));
+    TRY(dev_alloc(ctx, &ctx->d_rot, (group_variants ? B : 1) * ctx->R * ctx->S));
     TRY(dev_alloc(ctx, &ctx->d_key, B * ctx->N));
     if (ctx->mfma_sym) {
         TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->slices * ctx->sym_tiles * ctx->KSs * 1024));
@@ -1632,10 +1646,6 @@ int init_ctx(pink_hip_ctx *ctx)
         // rows beyond R and elements beyond the region must read as zero whoever fills the rest
         HIP_TRY(ctx, hipMemset(ctx->d_rotT, 0, B * ctx->Epad * ctx->Rpad * sizeof(uint32_t)));
     }
-    // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
-    // integer contexts, whenever the kernel keeps its base rotation in LDS.
-    ctx->fused_pack = ctx->use_lds && !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && ctx->D <= 4096 &&
-                      (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
     if (ctx->fused_pack) {
         const uint32_t D = ctx->D, DD = D * D;
         std::vector<uint32_t> symoff((size_t)8 * ctx->Epad, 0u);
