@@ -166,12 +166,15 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
             s_base[x * Dp + y] = base_pixel(img, I, D, i, cs, sn, x, y);
         }
         __syncthreads();
-        // (a mapper whose distance operand is packed below never reads the variants themselves)
+        // store_variants 0: none (a mapper whose distance operand is packed below never reads the variants);
+        // 1: all; 2: the base rotation and its quarter turn, of which the other six are row and column
+        // reversals (the update kernel reads them that way)
+        const uint32_t nf_st = store_variants == 2 ? 1u : nf, nq_st = store_variants == 2 ? min(nq, 2u) : nq;
         for (uint32_t p = threadIdx.x; p < (store_variants ? DD : 0u); p += blockDim.x) {
             const uint32_t x = p / D, y = p % D;
-            for (uint32_t f = 0; f < nf; ++f) {
+            for (uint32_t f = 0; f < nf_st; ++f) {
                 const uint32_t xs = f ? D - 1 - x : x;
-                for (uint32_t q = 0; q < nq; ++q) {
+                for (uint32_t q = 0; q < nq_st; ++q) {
                     uint32_t a, bb;
                     switch (q) {
                     case 0: a = xs; bb = y; break;
@@ -764,6 +767,28 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
 // Operand refresh of the integer GEMM path inside the update: the byte planes of the updated
 // elements (fragment order of mfma_int_gemm.inc) and the row norm |V|^2, accumulated per block
 // into `na_next` (zeroed by the distance kernel's finish step, which read the other buffer).
+// How the update kernel finds a variant when only two of a base rotation's eight symmetries are stored
+// (D = 0: every variant is stored).  Element counts stay below 2^24 (the base rotation fits LDS).
+struct VariantPair {
+    uint32_t D, num_rot, nrr;
+};
+
+// Quotient and remainder of a dividend below 2^24: the float reciprocal's estimate is within one of the
+// quotient and is corrected (a quarter of the instructions of the general 32-bit division).
+struct RcpDivisor {
+    uint32_t d;
+    float rcp;
+    __device__ explicit RcpDivisor(uint32_t d_) : d(d_), rcp(1.0f / (float)max(d_, 1u)) {}
+    __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
+    {
+        uint32_t e = (uint32_t)((float)n * rcp);
+        int rem = (int)(n - e * d);
+        if (rem < 0) { --e; rem += (int)d; }
+        else if ((uint32_t)rem >= d) { ++e; rem -= (int)d; }
+        q = e; r = (uint32_t)rem;
+    }
+};
+
 struct UpdatePlanes {
     signed char *Pa;            // null: not this path
     long long *na_next;
@@ -777,7 +802,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
                                                 uint32_t N, uint32_t S, uint32_t parts, uint32_t shift,
                                                 void *__restrict__ somP, const uint32_t *__restrict__ inv,
                                                 uint32_t Epad, float qfactor, UpdatePlanes up,
-                                                uint32_t *__restrict__ counts)
+                                                uint32_t *__restrict__ counts, VariantPair vp)
 {
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
@@ -795,7 +820,25 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         if (v < bv) { bv = v; bi = m; }        // ascending index per thread: first minimum kept
     }
     const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
+    // The variant: stored as such, or (vp.D != 0) read out of the stored base rotation (q even) or its
+    // quarter turn (q odd) with rows and/or columns reversed:
+    //   V(f, q)[x][y] = V(0, q & 1)[f ^ (q >> 1) ? D-1-x : x][q >> 1 ? D-1-y : y]
     const float *__restrict__ x = rot + (size_t)r * S;
+    uint32_t rev_x = 0, rev_y = 0;
+    if (vp.D) {
+        const uint32_t f = r >= vp.num_rot ? 1u : 0u, rem = r - f * vp.num_rot;
+        const uint32_t q = rem / vp.nrr, i = rem - q * vp.nrr;
+        x = rot + (size_t)((q & 1) * vp.nrr + i) * S;
+        rev_x = f ^ (q >> 1); rev_y = q >> 1;
+    }
+    const RcpDivisor by_DD(vp.D * vp.D), by_D(vp.D);
+    auto source = [&](uint32_t j) {
+        if (!vp.D) return j;
+        uint32_t c, p, px, py;
+        by_DD.divmod(j, c, p);
+        by_D.divmod(p, px, py);
+        return j - p + (rev_x ? vp.D - 1 - px : px) * vp.D + (rev_y ? vp.D - 1 - py : py);
+    };
     float *__restrict__ w = som + (size_t)n * S;
     const uint32_t chunk = (S + parts - 1) / parts;
     const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
@@ -807,7 +850,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
             const uint32_t j = jb + 256 * u;
             if (j < j1) {
                 wv[u] = w[j];
-                xv[u] = x[j];
+                xv[u] = x[source(j)];
                 kk[u] = inv ? inv[j] : 0xffffffffu;
             }
         }
@@ -922,6 +965,7 @@ __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__re
 // Host side
 // ---------------------------------------------------------------------------------
 struct EventPair { hipEvent_t a, b; int cls; };
+enum : uint32_t { kStoreNone = 0, kStoreAll = 1, kStorePair = 2 };
 
 }  // namespace
 
@@ -971,6 +1015,7 @@ struct pink_hip_ctx {
     uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
+    bool pair_variants = false;            // trainer: k_rotate stores two of the eight symmetries of a base rotation
     bool fused_som = false;                // integer GEMM trainer: k_update refreshes the SOM planes and norms itself
     uint32_t na_cur = 0;                   // which half of d_gna holds the norms of the current SOM operand
     int *d_na = nullptr, *d_nb = nullptr;
@@ -1145,8 +1190,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     return launch_check(ctx, "k_pack_som");
 }
 
-int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, bool store_variants = true)
+// store: kStoreNone, kStoreAll or kStorePair (see k_rotate)
+int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t store)
 {
+    const bool store_variants = store != kStoreNone;
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
     const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->Dp * sizeof(float) : 0;
@@ -1171,7 +1218,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, bool stor
 #define LAUNCH_ROTATE(P_)                                                                                          \
     hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
-                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store_variants ? 1u : 0u,                   \
+                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store,                   \
                        store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
@@ -1318,11 +1365,13 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
         up.na_next = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
         up.KS = ctx->gKS; up.Np = ctx->Np; up.u16 = ctx->cfg.ed_type == PINK_HIP_UINT16;
     }
+    VariantPair vp{};
+    if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
     hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
                        dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,
                        (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,
-                       is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts);
+                       is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp);
     if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
 }
@@ -1566,6 +1615,7 @@ int init_ctx(pink_hip_ctx *ctx)
                       (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
     // Float variants of a whole launch group: for the update kernel and for a separate packing kernel.
     // The other contexts keep room for one image (pink_hip_rotate).
+    ctx->pair_variants = ctx->trainer && ctx->fused_pack;
     const bool group_variants = ctx->trainer || !(ctx->mfma || ctx->mfma_sym || ctx->fused_pack);
 
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
@@ -1768,7 +1818,7 @@ int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
         return PINK_HIP_OK;
     }
     // the variants themselves are only read by the update kernel and by a separate packing kernel
-    TRY(run_rotate(ctx, dev_images, B, ctx->trainer || !ctx->fused_pack));
+    TRY(run_rotate(ctx, dev_images, B, ctx->fused_pack ? kStoreNone : kStoreAll));
     TRY(run_pack_rot(ctx, B));
     TRY(run_dist(ctx, 0, B));
     return PINK_HIP_OK;
@@ -1893,7 +1943,7 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
     // are produced for a group of images per launch.  Distance and update stay strictly sequential.
     for (uint32_t done = 0; done < n_images; done += ctx->Bcap) {
         const uint32_t B = std::min(ctx->Bcap, n_images - done);
-        TRY(run_rotate(ctx, dev_images + (size_t)done * ctx->isz, B));
+        TRY(run_rotate(ctx, dev_images + (size_t)done * ctx->isz, B, ctx->pair_variants ? kStorePair : kStoreAll));
         TRY(run_pack_rot(ctx, B));
         for (uint32_t b = 0; b < B; ++b) {
             TRY(run_dist(ctx, b, 1));
@@ -2087,7 +2137,7 @@ int pink_hip_rotate(pink_hip_ctx *ctx, const float *host_image, float *host_vari
     HIP_TRY(ctx, hipMalloc((void **)&d_img, (size_t)ctx->isz * sizeof(float)));
     hipError_t e = hipMemcpyAsync(d_img, host_image, (size_t)ctx->isz * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
     int rc = PINK_HIP_OK;
-    if (e == hipSuccess) rc = run_rotate(ctx, d_img, 1);
+    if (e == hipSuccess) rc = run_rotate(ctx, d_img, 1, kStoreAll);
     if (e == hipSuccess && rc == PINK_HIP_OK)
         e = hipMemcpyAsync(host_variants_out, ctx->d_rot, (size_t)ctx->R * ctx->S * sizeof(float), hipMemcpyDeviceToHost,
                            ctx->stream);
