@@ -121,7 +121,7 @@ __device__ __forceinline__ float base_pixel(const float *__restrict__ img, uint3
 // Operand packing fused into the rotation kernel (blocks that hold their base rotation in LDS):
 // the region of every variant goes straight from LDS into the distance kernel's operand, so the
 // variants are not read back.  symoff[sym * Epad + e] = channel << 24 | position in the base
-// rotation of region element e under symmetry sym = flip * 4 + quarter.
+// rotation of region element e under symmetry sym = flip * 4 + quarter (PACK 2 / 3: the position alone, 16 bits).
 //   PACK 1: float32 rows, opnd[(b * Rpad + k) * Epad + e]            (k = variant index)
 //   PACK 2 / 3: uint8 / uint16 byte planes in MFMA fragment order (see mfma_int_gemm.inc) and
 //               the row norms |V|^2; single channel only.
@@ -220,16 +220,17 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                 const uint32_t si = item % nsym, piece = item / nsym;   // neighbouring lanes: the adjacent rows of one piece
                 const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q;
                 const uint32_t r = i * nsym + si;             // operand row: the symmetries of a base rotation are adjacent
-                const uint4 *so4 = (const uint4 *)(pk.symoff + (size_t)sym * pk.Epad + piece * 16);
+                // (16-bit table entries here: one channel, and the base rotation has at most 16384 floats)
+                const uint2 *so4 = (const uint2 *)((const unsigned short *)pk.symoff + (size_t)sym * pk.Epad + piece * 16);
                 v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
                 int hh = 0, hl = 0, ll = 0;
 #pragma unroll
                 for (int w4 = 0; w4 < 4; ++w4) {
-                    const uint4 pv = so4[w4];
+                    const uint2 pv = so4[w4];
                     const uint32_t k0 = piece * 16 + w4 * 4;
                     const uint32_t valid = pk.E > k0 ? min(pk.E - k0, 4u) : 0u;
                     const uint32_t live = valid >= 4 ? 0xffffffffu : (1u << (8 * valid)) - 1u;
-                    const uint32_t q0 = clamp_q(pv.x), q1 = clamp_q(pv.y), q2 = clamp_q(pv.z), q3 = clamp_q(pv.w);
+                    const uint32_t q0 = clamp_q(pv.x & 0xffffu), q1 = clamp_q(pv.x >> 16), q2 = clamp_q(pv.y & 0xffffu), q3 = clamp_q(pv.y >> 16);
                     if constexpr (U16) {
                         const uint32_t w01 = q0 | (q1 << 16), w23 = q2 | (q3 << 16);
                         const int h = (int)((__builtin_amdgcn_perm(w23, w01, 0x07050301u) ^ 0x80808080u) & live);
@@ -1721,7 +1722,13 @@ int init_ctx(pink_hip_ctx *ctx)
         }
         if (ctx->base_hi <= ctx->base_lo) ctx->base_lo = ctx->base_hi = 0;       // empty region
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
-        HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, symoff.data(), symoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        if (ctx->gemm) {
+            // byte-plane packing reads 16-bit entries (single channel, positions below 16384)
+            std::vector<unsigned short> narrow(symoff.begin(), symoff.end());
+            HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, narrow.data(), narrow.size() * sizeof(unsigned short), hipMemcpyHostToDevice));
+        } else {
+            HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, symoff.data(), symoff.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        }
     }
     TRY(dev_alloc(ctx, &ctx->d_bmu_scratch, 1));
     TRY(dev_alloc(ctx, &ctx->d_counts, ctx->N));
