@@ -1036,8 +1036,6 @@ struct pink_hip_ctx {
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
 
-    uint32_t force_tn = 0;     // tuning aid: PINK_HIP_DIST_TN=1|2|4|8 overrides the neurons-per-wave choice
-
     bool profiling = false;
     std::vector<EventPair> events;
     std::vector<hipEvent_t> event_pool;
@@ -1290,7 +1288,6 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const uint32_t rblocks = ctx->Rpad / kWave;
     uint32_t tn = 4;
     while (tn > 1 && (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B < (size_t)4 * ctx->num_cu) tn >>= 1;
-    if (ctx->force_tn) tn = std::min(ctx->force_tn, 4u);
     const dim3 grid(rblocks, (ctx->N + 4 * tn - 1) / (4 * tn), B);
     const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
@@ -1878,10 +1875,6 @@ int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
     ctx->device = cfg->device;
     ctx->factor = cfg->ed_type == PINK_HIP_UINT8 ? 255u : cfg->ed_type == PINK_HIP_UINT16 ? 65535u : 1u;
     ctx->shift = cfg->ed_type == PINK_HIP_FLOAT ? 32u : 16u;
-    if (const char *e = getenv("PINK_HIP_DIST_TN")) {
-        const int v = atoi(e);
-        if (v == 1 || v == 2 || v == 4 || v == 8) ctx->force_tn = (uint32_t)v;
-    }
 
     int rc = init_ctx(ctx);
     if (rc != PINK_HIP_OK) {
