@@ -41,8 +41,8 @@ MEASURED_FMA_NOPACK_TFLOPS = 72.5
 # HBM bytes per image from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/cfg1_map_u8_hbm_traffic.txt),
 # scaled by the same counters' readings for a 256 MiB device-to-device copy (FETCH x2.0, WRITE x1.0).
 MEASURED_TRAFFIC_PER_IMAGE = {
-    ("cfg1", 3, "rotate"): 49.6e3 + 103.8e3,     # image + part of the geometry table read; units written
-    ("cfg1", 3, "distance"): 108.1e3 + 0.8e3,    # units read once; keys written
+    ("cfg1", 3, "rotate"): 49.2e3 + 103.8e3,     # image + part of the geometry table read; units written
+    ("cfg1", 3, "distance"): 107.3e3 + 0.8e3,    # units read once; keys written
 }
 
 

@@ -162,6 +162,26 @@ def test_train_one_call_per_image_equals_batched_call():
         assert np.array_equal(bits(a.get_som()), bits(b.get_som()))
 
 
+@pytest.mark.parametrize("name", ["cfg4", "cfg0"])
+def test_rotation_tap_between_training_calls(name):
+    # a trainer keeps two of a base rotation's eight symmetries; the tap asks for all of them in between
+    w = synthetic.WORKLOADS[name]
+    say("tap between training calls", name)
+    imgs = synthetic.images(w, 6)
+    som0 = synthetic.initial_som(w)
+    with synthetic.make_context(w) as a, synthetic.make_context(w) as b:
+        a.set_som(som0)
+        b.set_som(som0)
+        bm_a = a.train(imgs)
+        first = b.train(imgs[:3])
+        variants = b.rotate(imgs[5])
+        second = b.train(imgs[3:])
+        want = O.rotated_images(imgs[5], w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip)
+        assert np.array_equal(bits(variants), bits(want))
+        assert np.array_equal(bm_a, np.concatenate([first, second]))
+        assert np.array_equal(bits(a.get_som()), bits(b.get_som()))
+
+
 def test_reference_trainer_known_answers():
     # test/SelfOrganizingMapTest/Trainer.cpp:49-94 and test/CudaTest/update_neurons.cu:16-41
     F = capi.make_update_factors(capi.CARTESIAN, [2, 2], capi.GAUSSIAN, 1.1, 0.2, 0.0)
