@@ -1598,8 +1598,12 @@ int init_ctx(pink_hip_ctx *ctx)
             // 3 slices = 216 blocks beat 2 by 4 % and 4, a second round of blocks, by 30 %)
             uint32_t slices = std::max(1u, (uint32_t)ctx->num_cu / tiles);
             slices = std::min(slices, std::max(1u, ctx->gKS / 16));
-            // few k-steps per wave either way: one block per tile, which then finishes the tile itself
-            if ((ctx->gKS + 3) / 4 <= 8) slices = 1;
+            // Cutting k costs a second launch (about 5 us, the time of some 300 MFMAs): with fewer than 256
+            // MFMAs per wave one block per tile is faster, which then finishes the tile itself (measured at
+            // 64 k-steps: uint8, 64 MFMAs per wave, 47 k images/s in one slice against 43 k in four; uint16,
+            // 256 per wave, the break-even)
+            const uint32_t mfma_per_wave = ((ctx->gKS + 3) / 4) * (c.ed_type == PINK_HIP_UINT16 ? 16u : 4u);
+            if (mfma_per_wave < 256) slices = 1;
             ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
             ctx->gslices = (ctx->gKS + 4 * ctx->gks_per - 1) / (4 * ctx->gks_per);
         }
