@@ -54,7 +54,13 @@ def algorithmic_per_image(w, E, path):
     S, R, N = w.neuron_size, w.R, w.som_size
     nrr = max(w.num_rot // 4, 1)
     kp = -(-E // 64) * 64
-    rot_bytes = R * S * 4 + w.image_size * 4              # all variants written once, image read once
+    # k_rotate: image read once; a trainer's launch stores two of every base rotation's symmetries as
+    # float32 (the base rotation and its quarter turn, one when there is a single rotation) and the
+    # region of all R variants in the distance type; a mapper's launch stores the packed region only
+    stored = nrr * (2 if w.num_rot > 1 else 1) if w.mode == "train" else 0
+    rot_bytes = w.image_size * 4 + stored * S * 4 + R * E * elem
+    if w.ed_type != 0 and (path == 1 or w.channels > 1):     # integer distances on the vector ALU, or multi-channel
+        rot_bytes = w.image_size * 4 + R * S * 4          # all variants; a kernel of its own packs the region
     if path == 2:      # uint8 MFMA, symmetries on the image side: ceil(nrr/4) tiles of 32 rows + norms
         rot_bytes = w.image_size * 4 + -(-nrr // 4) * 32 * (kp + 4)
     elif path == 3:    # uint8 MFMA, symmetries on the SOM side: ceil(nrr/32) units of 32 rows + 1 KiB of norm entries
