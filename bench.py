@@ -65,12 +65,17 @@ def algorithmic_per_image(w, E, path):
         rot_bytes = w.image_size * 4 + -(-nrr // 4) * 32 * (kp + 4)
     elif path == 3:    # uint8 MFMA, symmetries on the SOM side: ceil(nrr/32) units of 32 rows + 1 KiB of norm entries
         rot_bytes = w.image_size * 4 + -(-nrr // 32) * (32 * kp + 1024)
+    # every operand element read once: all R variants and the N neurons, or, where the symmetries sit on
+    # the SOM side (operand in registers), the units of the base rotations the rotation kernel wrote + the keys
+    dist_bytes = (R + N) * E * elem
+    if path == 3:
+        dist_bytes = -(-nrr // 32) * (32 * kp + 1024) + N * 8
     return {
         "rotate": {"bytes": rot_bytes},
         # region of every variant read as float32 and written in the distance type
         "pack": {"bytes": R * E * (4 + elem)},
-        # every operand element read once; one subtract-square-accumulate = 2 operations
-        "distance": {"bytes": (R + N) * E * elem, "ops": 2 * N * R * E},
+        # one subtract-square-accumulate = 2 operations
+        "distance": {"bytes": dist_bytes, "ops": 2 * N * R * E},
         # SOM read + written, one variant read per neuron
         "update": {"bytes": 3 * N * S * 4},
         "finalize": {"bytes": N * 16},
@@ -240,7 +245,7 @@ def main():
             dist["frac_of_measured_nopack_fma"] = round(dist["ops_per_s"] / 1e12 / MEASURED_FMA_NOPACK_TFLOPS, 5)
         else:
             dist["frac_of_int8_mfma_5POPs"] = round(dist["ops_per_s"] / 1e12 / MFMA_INT8_PEAK_TOPS, 5)
-            dist["hbm_frac_survey_bytes"] = round(alg["distance"]["bytes"] * d_per_s / 1e9 / HBM_PEAK_GBS, 5)
+            dist["hbm_frac_algorithmic_bytes"] = round(alg["distance"]["bytes"] * d_per_s / 1e9 / HBM_PEAK_GBS, 5)
         dist["ops_per_s"] = round(dist["ops_per_s"] / 1e12, 3)
         roofline["distance_kernel"] = dist
     r_launches, r_ms = times["rotate"]
