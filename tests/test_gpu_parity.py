@@ -372,6 +372,28 @@ def test_train_over_shapes(N, C_, I, D, nrot, flip, ed, shape_, ed_type, n):
     assert np.array_equal(bits(d1), bits(d2)) and np.array_equal(ssd1, ssd2) and np.array_equal(best1, best2)
 
 
+@pytest.mark.parametrize("N,ed_type", [(9, capi.FLOAT), (9, capi.UINT8), (530, capi.UINT8)])
+def test_train_with_any_factor_matrix(N, ed_type):
+    # the C interface takes any N x N matrix, not only the symmetric ones that a distance functor gives
+    say("train, factor matrix", N, ed_type)
+    C_, I, D, nrot, flip, ed, n = 1, 12, 8, 4, True, 6, 3
+    rng = np.random.default_rng(N + ed_type)
+    som0 = rng.random((N, C_ * D * D), dtype=np.float32)
+    imgs = rng.random((n, C_, I, I), dtype=np.float32)
+    F = rng.random((N, N), dtype=np.float32) * np.float32(0.5)
+    F[rng.random((N, N)) < 0.3] = 0.0
+    assert not np.array_equal(F, F.T)
+    s = O.shape(N, C_, I, D, nrot, flip, ed, capi.QUADRATIC, ed_type)
+    want = som0.copy()
+    obmu = O.train(s, want, imgs, F)
+    with capi.Context(N, C_, I, D, nrot, flip, ed, capi.QUADRATIC, ed_type, F) as ctx:
+        ctx.set_som(som0)
+        bmu = ctx.train(imgs)
+        som = ctx.get_som()
+    assert np.array_equal(bmu, obmu)
+    assert np.array_equal(bits(som), bits(want))
+
+
 def test_reference_mapper_known_answers():
     # test/CudaTest/mapper.cu:115-119 in float, uint8 and uint16; circular_ed.cu:23-53
     for som_dim, nd, idim, ed, nrot, flip in [(1, 2, 2, 2, 1, False), (1, 3, 3, 2, 1, False), (1, 3, 3, 2, 360, False),
