@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 ROT_SHAPES = [
-    # C, I, D, num_rot, flip        (cfg = BASELINE config shapes, then the odd ones of
+    # C, I, D, num_rot, flip        (the benchmark configurations, then the odd ones of
     #                                test/CudaTest/compare_trainer_cpu.cu:81-98)
     (1, 64, 44, 360, True),         # cfg 0 / 1
     (1, 150, 106, 360, True),       # cfg 2
