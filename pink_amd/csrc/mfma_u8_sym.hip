@@ -934,8 +934,10 @@ template <int G>
 hipError_t launch_rotpack(hipStream_t stream, const RotpackArgs &g, bool configure_only)
 {
     const size_t lds = (size_t)G * lds_image_bytes(g.C, g.I);
+    // (the limit is per kernel, not per context: the most that any context may ask of this instantiation)
     if (configure_only)
-        return hipFuncSetAttribute((const void *)k_rotpack_sym_u8<G>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        return hipFuncSetAttribute((const void *)k_rotpack_sym_u8<G>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   G == 1 ? 150 * 1024 : 76 * 1024);
     const uint32_t groups = (g.B + G - 1) / G;
     const uint32_t blocks = ((groups + 7) / 8) * 8 * g.RTP;           // 8 groups per span of ids, see the kernel
     hipLaunchKernelGGL(k_rotpack_sym_u8<G>, dim3(blocks), dim3(G >= 4 ? 512 : 256), lds, stream, g.images, (v4i *)g.Pb, g.tab_idx,

@@ -966,6 +966,7 @@ __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__re
 // Host side
 // ---------------------------------------------------------------------------------
 struct EventPair { hipEvent_t a, b; int cls; };
+constexpr size_t kRotateLdsMax = 158 * 1024;
 enum : uint32_t { kStoreNone = 0, kStoreAll = 1, kStorePair = 2 };
 
 }  // namespace
@@ -997,7 +998,7 @@ struct pink_hip_ctx {
     // uint8 mapping on the matrix cores
     bool mfma = false;
     uint32_t KS = 0, RT = 0, NT = 0, n_need = 0, nrr_eff = 1;
-    size_t lds_dist = 0, lds_rotpack = 0;
+    size_t lds_dist = 0, lds_rotpack = 0, lds_max = 0;
     int num_cu = 256;
     signed char *d_Pa = nullptr, *d_Pb = nullptr;
     void *d_rtab = nullptr;                // geometry table of the base rotations (symmetric MFMA path)
@@ -1445,6 +1446,7 @@ int init_ctx(pink_hip_ctx *ctx)
         HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
         ctx->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
         const size_t lds_max = std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024) - 1024;
+        ctx->lds_max = lds_max;
         ctx->nrr_eff = std::max(ctx->nrr, 1u);
         ctx->KS = ctx->Epad / 32;
         ctx->NT = (ctx->N + 31) / 32;
@@ -1572,11 +1574,12 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, &ctx->d_need, need.size()));
         HIP_TRY(ctx, hipMemcpy(ctx->d_poff, poff.data(), poff.size() * sizeof(unsigned short), hipMemcpyHostToDevice));
         HIP_TRY(ctx, hipMemcpy(ctx->d_need, need.data(), need.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        // (limits are per kernel, not per context: the most that any context may ask)
         HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotpack_u8, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)ctx->lds_rotpack));
+                                         (int)ctx->lds_max));
         const void *fn = ctx->NT == 1 ? (const void *)k_dist_mfma_u8<1> : ctx->NT == 2 ? (const void *)k_dist_mfma_u8<2>
                        : ctx->NT == 3 ? (const void *)k_dist_mfma_u8<3> : (const void *)k_dist_mfma_u8<4>;
-        HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_dist));
+        HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_max));
     }
 
     // Integer distances as a split-k int8 GEMM: all that is left of the integer modes.  Small
@@ -1610,7 +1613,15 @@ int init_ctx(pink_hip_ctx *ctx)
     }
 
     ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
-    ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= 64 * 1024;
+    // the base rotation of a block lives in LDS: up to 158 of the CU's 160 KB (neurons up to 199 pixels wide)
+    ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax;
+    if (ctx->use_lds) {
+        const int lds = (int)kRotateLdsMax;          // per kernel, not per context: the most any context may ask
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    }
     // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
     // integer contexts, whenever the kernel keeps its base rotation in LDS.
     ctx->fused_pack = ctx->use_lds && !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && ctx->D <= 4096 &&

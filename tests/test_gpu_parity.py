@@ -30,7 +30,8 @@ ROT_SHAPES = [
     (1, 64, 44, 360, True), (1, 150, 106, 360, True), (3, 100, 70, 180, True), (1, 28, 28, 4, True),
     (1, 64, 45, 360, True), (1, 64, 100, 360, True), (1, 124, 91, 360, True), (2, 17, 24, 16, False),
     (1, 2, 4, 1, False), (1, 4, 2, 8, True), (1, 5, 3, 360, False), (3, 9, 9, 1, True),
-    (1, 200, 141, 8, True),     # 141*141*4 B > 64 KiB: the no-LDS path
+    (1, 200, 141, 8, True),     # a base rotation of 78 KiB in LDS
+    (1, 290, 205, 8, True),     # 205*205*4 B > 158 KiB: the path without an LDS tile
 ]
 
 
@@ -342,8 +343,10 @@ FUSED_TRAIN_SHAPES = [
     (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.FLOAT, 4),        # three channels, float32 rows from the rotation kernel
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.FLOAT, 3),           # region repeats channel 0 (CPU rule): no inverse table
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.UINT16, 3),
-    (4, 1, 200, 150, 8, True, 100, capi.CIRCULAR, capi.UINT8, 2),     # neurons too large for the rotation kernel's LDS tile
+    (4, 1, 200, 150, 8, True, 100, capi.CIRCULAR, capi.UINT8, 2),     # a large LDS tile in the rotation kernel
     (3, 1, 160, 129, 4, True, 128, capi.QUADRATIC, capi.FLOAT, 2),
+    (4, 1, 290, 205, 8, True, 100, capi.CIRCULAR, capi.UINT8, 2),     # neurons too large for the rotation kernel's LDS tile
+    (3, 1, 280, 201, 4, True, 128, capi.QUADRATIC, capi.FLOAT, 2),
     (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
 ]
 
@@ -392,6 +395,31 @@ def test_train_with_any_factor_matrix(N, ed_type):
         som = ctx.get_som()
     assert np.array_equal(bmu, obmu)
     assert np.array_equal(bits(som), bits(want))
+
+
+def test_contexts_of_different_sizes_side_by_side():
+    # LDS limits are set per kernel, not per context: a context created later with smaller images must
+    # not take away what an earlier one needs (uint8 mappers of 150 and 100 pixels, trainers of 181 and 44)
+    say("contexts side by side")
+    rng = np.random.default_rng(77)
+    made = []
+    for (I, D, ed, et, F) in ((150, 30, 20, capi.UINT8, None), (100, 30, 20, capi.UINT8, None),
+                              (128, 181, 90, capi.UINT16, capi.make_update_factors(capi.CARTESIAN, [4], capi.GAUSSIAN, 1.0, 0.5)),
+                              (64, 44, 32, capi.UINT16, capi.make_update_factors(capi.CARTESIAN, [4], capi.GAUSSIAN, 1.0, 0.5))):
+        ctx = capi.Context(4, 1, I, D, 8, True, ed, capi.QUADRATIC, et, F)
+        som = rng.random((4, D * D), dtype=np.float32)
+        img = rng.random((1, I, I), dtype=np.float32)
+        ctx.set_som(som)
+        made.append((ctx, som, img, I, D, ed, et))
+    try:
+        for ctx, som, img, I, D, ed, et in made:          # the first contexts run after the last was created
+            s = O.shape(4, 1, I, D, 8, True, ed, capi.QUADRATIC, et)
+            od, ossd, obest = O.distance_matrix(s, som, O.rotated_images(img, 1, I, D, 8, True))
+            d, ssd, best = ctx.distance(img)
+            assert np.array_equal(ssd, ossd) and np.array_equal(best, obest)
+    finally:
+        for m in made:
+            m[0].close()
 
 
 def test_reference_mapper_known_answers():
