@@ -107,6 +107,22 @@ __device__ __forceinline__ float base_pixel(const float *__restrict__ img, uint3
     return __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
 }
 
+// Quotient and remainder of a dividend below 2^24: the float reciprocal's estimate is within one of the
+// quotient and is corrected (a quarter of the instructions of the general 32-bit division).
+struct RcpDivisor {
+    uint32_t d;
+    float rcp;
+    __device__ explicit RcpDivisor(uint32_t d_) : d(d_), rcp(1.0f / (float)max(d_, 1u)) {}
+    __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
+    {
+        uint32_t e = (uint32_t)((float)n * rcp);
+        int rem = (int)(n - e * d);
+        if (rem < 0) { --e; rem += (int)d; }
+        else if ((uint32_t)rem >= d) { ++e; rem -= (int)d; }
+        q = e; r = (uint32_t)rem;
+    }
+};
+
 // ---------------------------------------------------------------------------------
 // Rotation: all num_rot * (flip ? 2 : 1) variants of a batch of images.
 // Block (i, c, b) computes base rotation i of channel c of image b once, keeps it in
@@ -132,12 +148,12 @@ struct PackArgs {
     uint32_t E, Epad, rows_pad, KS;
 };
 
-template <int PACK>
+template <int PACK, bool use_lds>
 __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
-                                                uint32_t use_flip, uint32_t use_lds, uint32_t Dp, PackArgs pk,
+                                                uint32_t use_flip, uint32_t Dp, PackArgs pk,
                                                 uint32_t store_variants, uint32_t lo, uint32_t hi)
 {
     // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
@@ -157,7 +173,23 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         for (uint32_t n = threadIdx.x; n < N; n += blockDim.x) key[(size_t)b * N + n] = ~0ull;
     if (PACK >= 2 && threadIdx.x < 8) s_norm[threadIdx.x] = 0;
 
-    if (use_lds) {
+    // Pixel (a, bb) of the base rotation: out of the LDS tile, or, for neurons too large for one,
+    // computed where it is needed (every stored or packed element then costs one interpolation, which
+    // is cheaper than strided stores of values computed once).  Positions arrive as a * Dp + bb.
+    auto sample = [&](uint32_t a, uint32_t bb) {
+        if constexpr (use_lds) return s_base[a * Dp + bb];
+        else return base_pixel(img, I, D, i, cs, sn, a, bb);
+    };
+    const RcpDivisor by_Dp(Dp);
+    auto sample_at = [&](uint32_t po) {
+        if constexpr (use_lds) return s_base[po];
+        else {
+            uint32_t a, bb;
+            by_Dp.divmod(po, a, bb);
+            return base_pixel(img, I, D, i, cs, sn, a, bb);
+        }
+    };
+    if constexpr (use_lds) {
         // rows and columns [lo, hi) of the base rotation: all of it, or, when only the packed operand is
         // wanted, the square that the region reaches under the eight symmetries
         const uint32_t side = hi - lo;
@@ -166,6 +198,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
             s_base[x * Dp + y] = base_pixel(img, I, D, i, cs, sn, x, y);
         }
         __syncthreads();
+    }
+    {
         // store_variants 0: none (a mapper whose distance operand is packed below never reads the variants);
         // 1: all; 2: the base rotation and its quarter turn, of which the other six are row and column
         // reversals (the update kernel reads them that way)
@@ -183,7 +217,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     default: a = y; bb = D - 1 - xs; break;
                     }
                     const uint32_t k = f * num_rot + q * nrr + i;
-                    out[((size_t)k * C + c) * DD + p] = s_base[a * Dp + bb];
+                    out[((size_t)k * C + c) * DD + p] = sample(a, bb);
                 }
             }
         }
@@ -195,7 +229,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     float *row = opnd + (size_t)(f * num_rot + q * nrr + i) * pk.Epad;
                     for (uint32_t e = threadIdx.x; e < pk.E; e += blockDim.x) {
                         const uint32_t po = so[e];
-                        if ((po >> 24) == c) row[e] = s_base[po & 0xffffffu];
+                        if ((po >> 24) == c) row[e] = sample_at(po & 0xffffffu);
                     }
                 }
         } else if constexpr (PACK >= 2) {
@@ -213,24 +247,32 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
             v4i *P = (v4i *)pk.opnd + (size_t)b * planes * plane_stride;
             const uint32_t pieces = pk.KS * 2, nsym = nf * nq;
             auto clamp_q = [&](uint32_t po) {
-                const float v = fminf(fmaxf(__fmul_rn(s_base[po], factor), 0.0f), factor);   // NaN -> 0
+                const float v = fminf(fmaxf(__fmul_rn(sample_at(po), factor), 0.0f), factor);   // NaN -> 0
                 return (uint32_t)v;
             };
             for (uint32_t item = threadIdx.x; item < nsym * pieces; item += blockDim.x) {
                 const uint32_t si = item % nsym, piece = item / nsym;   // neighbouring lanes: the adjacent rows of one piece
                 const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q;
                 const uint32_t r = i * nsym + si;             // operand row: the symmetries of a base rotation are adjacent
-                // (16-bit table entries here: one channel, and the base rotation has at most 16384 floats)
+                // (16-bit table entries with an LDS tile: one channel, at most 40 000 floats; 32-bit without)
                 const uint2 *so4 = (const uint2 *)((const unsigned short *)pk.symoff + (size_t)sym * pk.Epad + piece * 16);
+                const uint4 *so4w = (const uint4 *)(pk.symoff + (size_t)sym * pk.Epad + piece * 16);
                 v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
                 int hh = 0, hl = 0, ll = 0;
 #pragma unroll
                 for (int w4 = 0; w4 < 4; ++w4) {
-                    const uint2 pv = so4[w4];
+                    uint32_t p0, p1, p2, p3;
+                    if constexpr (use_lds) {
+                        const uint2 pv = so4[w4];
+                        p0 = pv.x & 0xffffu; p1 = pv.x >> 16; p2 = pv.y & 0xffffu; p3 = pv.y >> 16;
+                    } else {
+                        const uint4 pv = so4w[w4];
+                        p0 = pv.x; p1 = pv.y; p2 = pv.z; p3 = pv.w;
+                    }
                     const uint32_t k0 = piece * 16 + w4 * 4;
                     const uint32_t valid = pk.E > k0 ? min(pk.E - k0, 4u) : 0u;
                     const uint32_t live = valid >= 4 ? 0xffffffffu : (1u << (8 * valid)) - 1u;
-                    const uint32_t q0 = clamp_q(pv.x & 0xffffu), q1 = clamp_q(pv.x >> 16), q2 = clamp_q(pv.y & 0xffffu), q3 = clamp_q(pv.y >> 16);
+                    const uint32_t q0 = clamp_q(p0), q1 = clamp_q(p1), q2 = clamp_q(p2), q3 = clamp_q(p3);
                     if constexpr (U16) {
                         const uint32_t w01 = q0 | (q1 << 16), w23 = q2 | (q3 << 16);
                         const int h = (int)((__builtin_amdgcn_perm(w23, w01, 0x07050301u) ^ 0x80808080u) & live);
@@ -256,26 +298,6 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                 const uint32_t f = threadIdx.x >> 2, q = threadIdx.x & 3;
                 if (f < nf && q < nq)
                     pk.norm[(size_t)b * pk.rows_pad + i * nsym + f * nq + q] = (long long)s_norm[threadIdx.x];
-            }
-        }
-    } else {
-        // Neurons too large for LDS: compute each base pixel once and scatter it.
-        for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
-            const uint32_t a = p / D, bb = p % D;
-            const float v = base_pixel(img, I, D, i, cs, sn, a, bb);
-            for (uint32_t q = 0; q < nq; ++q) {
-                uint32_t x, y;
-                switch (q) {
-                case 0: x = a; y = bb; break;
-                case 1: x = bb; y = D - 1 - a; break;
-                case 2: x = D - 1 - a; y = D - 1 - bb; break;
-                default: x = D - 1 - bb; y = a; break;
-                }
-                for (uint32_t f = 0; f < nf; ++f) {
-                    const uint32_t xf = f ? D - 1 - x : x;
-                    const uint32_t k = f * num_rot + q * nrr + i;
-                    out[((size_t)k * C + c) * DD + xf * D + y] = v;
-                }
             }
         }
     }
@@ -774,22 +796,6 @@ struct VariantPair {
     uint32_t D, num_rot, nrr;
 };
 
-// Quotient and remainder of a dividend below 2^24: the float reciprocal's estimate is within one of the
-// quotient and is corrected (a quarter of the instructions of the general 32-bit division).
-struct RcpDivisor {
-    uint32_t d;
-    float rcp;
-    __device__ explicit RcpDivisor(uint32_t d_) : d(d_), rcp(1.0f / (float)max(d_, 1u)) {}
-    __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
-    {
-        uint32_t e = (uint32_t)((float)n * rcp);
-        int rem = (int)(n - e * d);
-        if (rem < 0) { --e; rem += (int)d; }
-        else if ((uint32_t)rem >= d) { ++e; rem -= (int)d; }
-        q = e; r = (uint32_t)rem;
-    }
-};
-
 struct UpdatePlanes {
     signed char *Pa;            // null: not this path
     long long *na_next;
@@ -1215,11 +1221,16 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
             pk.opnd = ctx->d_rotT; pk.rows_pad = ctx->Rpad;
         }
     }
-#define LAUNCH_ROTATE(P_)                                                                                          \
-    hipLaunchKernelGGL(k_rotate<P_>, grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
+#define LAUNCH_ROTATE_(P_, L_)                                                                                     \
+    hipLaunchKernelGGL((k_rotate<P_, L_>), grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
-                       ctx->use_lds ? 1u : 0u, ctx->Dp, pk, store,                   \
+                       ctx->Dp, pk, store,                   \
                        store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi)
+#define LAUNCH_ROTATE(P_)                         \
+    do {                                          \
+        if (ctx->use_lds) LAUNCH_ROTATE_(P_, true);  \
+        else LAUNCH_ROTATE_(P_, false);           \
+    } while (0)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
     case 2: LAUNCH_ROTATE(2); break;
@@ -1227,6 +1238,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
     default: LAUNCH_ROTATE(0); break;
     }
 #undef LAUNCH_ROTATE
+#undef LAUNCH_ROTATE_
     return launch_check(ctx, "k_rotate");
 }
 
@@ -1617,18 +1629,18 @@ int init_ctx(pink_hip_ctx *ctx)
     ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax;
     if (ctx->use_lds) {
         const int lds = (int)kRotateLdsMax;          // per kernel, not per context: the most any context may ask
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     }
     // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
     // integer contexts, whenever the kernel keeps its base rotation in LDS.
-    ctx->fused_pack = ctx->use_lds && !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && ctx->D <= 4096 &&
+    ctx->fused_pack = !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && (size_t)ctx->D * ctx->Dp < ((size_t)1 << 24) &&
                       (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
     // Float variants of a whole launch group: for the update kernel and for a separate packing kernel.
     // The other contexts keep room for one image (pink_hip_rotate).
-    ctx->pair_variants = ctx->trainer && ctx->fused_pack;
+    ctx->pair_variants = ctx->trainer && ctx->fused_pack && ctx->S < (1u << 24);   // (the update kernel's divisions)
     const bool group_variants = ctx->trainer || !(ctx->mfma || ctx->mfma_sym || ctx->fused_pack);
 
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
@@ -1734,8 +1746,8 @@ int init_ctx(pink_hip_ctx *ctx)
         }
         if (ctx->base_hi <= ctx->base_lo) ctx->base_lo = ctx->base_hi = 0;       // empty region
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
-        if (ctx->gemm) {
-            // byte-plane packing reads 16-bit entries (single channel, positions below 16384)
+        if (ctx->gemm && ctx->use_lds) {
+            // byte-plane packing out of an LDS tile reads 16-bit entries (single channel, positions below 40 000)
             std::vector<unsigned short> narrow(symoff.begin(), symoff.end());
             HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, narrow.data(), narrow.size() * sizeof(unsigned short), hipMemcpyHostToDevice));
         } else {
