@@ -148,7 +148,7 @@ struct PackArgs {
     uint32_t E, Epad, rows_pad, KS;
 };
 
-template <int PACK, bool use_lds>
+template <int PACK, int TILE>
 __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ images, float *__restrict__ rot,
                                                 const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                 unsigned long long *__restrict__ key, uint32_t N,
@@ -158,8 +158,11 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
 {
     // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
     // stride keeps those reads in different banks (a stride of 64 would put all of them into one)
+    // TILE 1: as described; 2: neurons too large for that, the image channel is in LDS instead and every
+    // element is interpolated out of it where it is needed; 0: neither fits, the image is read from memory
     extern __shared__ float s_base[];
     __shared__ unsigned long long s_norm[8];
+    constexpr bool use_lds = TILE == 1;
     const uint32_t i = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
     const uint32_t nrr = num_rot / 4;
     const uint32_t R = num_rot * (use_flip ? 2u : 1u);
@@ -177,7 +180,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     // computed where it is needed (every stored or packed element then costs one interpolation, which
     // is cheaper than strided stores of values computed once).  Positions arrive as a * Dp + bb.
     auto sample = [&](uint32_t a, uint32_t bb) {
-        if constexpr (use_lds) return s_base[a * Dp + bb];
+        if constexpr (TILE == 1) return s_base[a * Dp + bb];
+        else if constexpr (TILE == 2) return base_pixel(s_base, I, D, i, cs, sn, a, bb);
         else return base_pixel(img, I, D, i, cs, sn, a, bb);
     };
     const RcpDivisor by_Dp(Dp);
@@ -186,9 +190,13 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         else {
             uint32_t a, bb;
             by_Dp.divmod(po, a, bb);
-            return base_pixel(img, I, D, i, cs, sn, a, bb);
+            return sample(a, bb);
         }
     };
+    if constexpr (TILE == 2) {
+        for (uint32_t p = threadIdx.x; p < I * I; p += blockDim.x) s_base[p] = img[p];
+        __syncthreads();
+    }
     if constexpr (use_lds) {
         // rows and columns [lo, hi) of the base rotation: all of it, or, when only the packed operand is
         // wanted, the square that the region reaches under the eight symmetries
@@ -987,7 +995,8 @@ struct pink_hip_ctx {
     uint32_t shift = 32;       // key = value << shift | rotation
     uint32_t factor = 1;       // 255 / 65535 in the integer modes
     bool trainer = false;
-    bool use_lds = true;
+    bool use_lds = true;       // the rotation kernel keeps a block's base rotation in LDS
+    bool image_lds = false;    // ... or, neurons too large for that, the image channel
     int device = 0;
     hipStream_t stream = nullptr;
 
@@ -1202,7 +1211,8 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
     const bool store_variants = store != kStoreNone;
     Timed t(ctx, kClsRotate);
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
-    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->Dp * sizeof(float) : 0;
+    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->Dp * sizeof(float)
+                     : ctx->image_lds ? (size_t)ctx->I * ctx->I * sizeof(float) : 0;
     // about four neuron pixels per thread: large neurons get large blocks, whose many waves per LDS
     // footprint hide the latency of the gathers (measured: 1024 threads 35 % faster than 256 at 3 x 70 x 70)
     uint32_t threads = 256;
@@ -1228,8 +1238,9 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
                        store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi)
 #define LAUNCH_ROTATE(P_)                         \
     do {                                          \
-        if (ctx->use_lds) LAUNCH_ROTATE_(P_, true);  \
-        else LAUNCH_ROTATE_(P_, false);           \
+        if (ctx->use_lds) LAUNCH_ROTATE_(P_, 1);  \
+        else if (ctx->image_lds) LAUNCH_ROTATE_(P_, 2); \
+        else LAUNCH_ROTATE_(P_, 0);               \
     } while (0)
     switch (pack) {
     case 1: LAUNCH_ROTATE(1); break;
@@ -1627,12 +1638,17 @@ int init_ctx(pink_hip_ctx *ctx)
     ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
     // the base rotation of a block lives in LDS: up to 158 of the CU's 160 KB (neurons up to 199 pixels wide)
     ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax;
-    if (ctx->use_lds) {
+    ctx->image_lds = !ctx->use_lds && (size_t)ctx->I * ctx->I * sizeof(float) <= kRotateLdsMax;
+    {
         const int lds = (int)kRotateLdsMax;          // per kernel, not per context: the most any context may ask
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<0, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_rotate<3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     }
     // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
     // integer contexts, whenever the kernel keeps its base rotation in LDS.

@@ -31,7 +31,9 @@ ROT_SHAPES = [
     (1, 64, 45, 360, True), (1, 64, 100, 360, True), (1, 124, 91, 360, True), (2, 17, 24, 16, False),
     (1, 2, 4, 1, False), (1, 4, 2, 8, True), (1, 5, 3, 360, False), (3, 9, 9, 1, True),
     (1, 200, 141, 8, True),     # a base rotation of 78 KiB in LDS
-    (1, 290, 205, 8, True),     # 205*205*4 B > 158 KiB: the path without an LDS tile
+    (1, 290, 205, 8, True),     # 205*205*4 B > 158 KiB and so is the image: nothing in LDS
+    (1, 150, 205, 16, True),    # the image in LDS instead of the base rotation
+    (2, 160, 226, 8, False),
 ]
 
 
@@ -68,6 +70,9 @@ DIST_SHAPES = [
     (5, 1, 8, 8, 1, True, 5, capi.QUADRATIC),
     (331, 1, 150, 106, 360, True, 75, capi.CIRCULAR),     # cfg 2
     (1600, 3, 100, 70, 180, True, 50, capi.QUADRATIC),    # cfg 3
+    (5, 1, 160, 226, 8, True, 113, capi.QUADRATIC),       # neurons too large for an LDS tile: the image in LDS
+    (5, 1, 290, 205, 8, True, 40, capi.CIRCULAR),         # ... nothing in LDS
+    (5, 1, 128, 181, 16, True, 90, capi.QUADRATIC),       # a 128 KiB base rotation in LDS
 ]
 
 
@@ -347,6 +352,9 @@ FUSED_TRAIN_SHAPES = [
     (3, 1, 160, 129, 4, True, 128, capi.QUADRATIC, capi.FLOAT, 2),
     (4, 1, 290, 205, 8, True, 100, capi.CIRCULAR, capi.UINT8, 2),     # neurons too large for the rotation kernel's LDS tile
     (3, 1, 280, 201, 4, True, 128, capi.QUADRATIC, capi.FLOAT, 2),
+    (4, 1, 160, 226, 8, True, 113, capi.QUADRATIC, capi.UINT8, 2),    # ... but the image fits: interpolated out of LDS
+    (3, 1, 160, 226, 8, True, 113, capi.CIRCULAR, capi.UINT16, 2),
+    (3, 1, 150, 201, 8, True, 100, capi.QUADRATIC, capi.FLOAT, 2),
     (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
 ]
 
