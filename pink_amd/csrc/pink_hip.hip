@@ -146,6 +146,7 @@ struct PackArgs {
     void *opnd;            // float rows, or byte planes
     long long *norm;       // integer modes: [b][Rp]
     uint32_t E, Epad, rows_pad, KS;
+    uint32_t wide;         // integer modes: table entries of 32 bits (else 16)
 };
 
 template <int PACK, int TILE>
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                                                 unsigned long long *__restrict__ key, uint32_t N,
                                                 uint32_t C, uint32_t I, uint32_t D, uint32_t num_rot,
                                                 uint32_t use_flip, uint32_t Dp, PackArgs pk,
-                                                uint32_t store_variants, uint32_t lo, uint32_t hi)
+                                                uint32_t store_variants, uint32_t lo, uint32_t hi, uint32_t nch)
 {
     // the base rotation, rows of Dp floats (odd): the quarter turns read it along columns, and an odd
     // stride keeps those reads in different banks (a stride of 64 would put all of them into one)
@@ -163,7 +164,10 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     extern __shared__ float s_base[];
     __shared__ unsigned long long s_norm[8];
     constexpr bool use_lds = TILE == 1;
-    const uint32_t i = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
+    // a block holds the base rotation of nch channels (TILE 1: one, or all of them when they fit LDS
+    // together, which lets the byte planes of multi-channel data be packed here; else one), tile after tile
+    const uint32_t i = blockIdx.x, c = blockIdx.y * nch, b = blockIdx.z;
+    const uint32_t tile = D * Dp;
     const uint32_t nrr = num_rot / 4;
     const uint32_t R = num_rot * (use_flip ? 2u : 1u);
     const uint32_t DD = D * D;
@@ -179,18 +183,19 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     // Pixel (a, bb) of the base rotation: out of the LDS tile, or, for neurons too large for one,
     // computed where it is needed (every stored or packed element then costs one interpolation, which
     // is cheaper than strided stores of values computed once).  Positions arrive as a * Dp + bb.
-    auto sample = [&](uint32_t a, uint32_t bb) {
-        if constexpr (TILE == 1) return s_base[a * Dp + bb];
+    // (cc = channel within the block; TILE 0 and 2 have one channel per block)
+    auto sample = [&](uint32_t cc, uint32_t a, uint32_t bb) {
+        if constexpr (TILE == 1) return s_base[cc * tile + a * Dp + bb];
         else if constexpr (TILE == 2) return base_pixel(s_base, I, D, i, cs, sn, a, bb);
         else return base_pixel(img, I, D, i, cs, sn, a, bb);
     };
     const RcpDivisor by_Dp(Dp);
-    auto sample_at = [&](uint32_t po) {
+    auto sample_at = [&](uint32_t po) {               // po: position in the block's LDS tiles
         if constexpr (use_lds) return s_base[po];
         else {
             uint32_t a, bb;
             by_Dp.divmod(po, a, bb);
-            return sample(a, bb);
+            return sample(0, a, bb);
         }
     };
     if constexpr (TILE == 2) {
@@ -201,10 +206,11 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         // rows and columns [lo, hi) of the base rotation: all of it, or, when only the packed operand is
         // wanted, the square that the region reaches under the eight symmetries
         const uint32_t side = hi - lo;
-        for (uint32_t p = threadIdx.x; p < side * side; p += blockDim.x) {
-            const uint32_t x = lo + p / side, y = lo + p % side;
-            s_base[x * Dp + y] = base_pixel(img, I, D, i, cs, sn, x, y);
-        }
+        for (uint32_t cc = 0; cc < nch; ++cc)
+            for (uint32_t p = threadIdx.x; p < side * side; p += blockDim.x) {
+                const uint32_t x = lo + p / side, y = lo + p % side;
+                s_base[cc * tile + x * Dp + y] = base_pixel(img + (size_t)cc * I * I, I, D, i, cs, sn, x, y);
+            }
         __syncthreads();
     }
     {
@@ -225,7 +231,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     default: a = y; bb = D - 1 - xs; break;
                     }
                     const uint32_t k = f * num_rot + q * nrr + i;
-                    out[((size_t)k * C + c) * DD + p] = sample(a, bb);
+                    for (uint32_t cc = 0; cc < nch; ++cc) out[((size_t)k * C + c + cc) * DD + p] = sample(cc, a, bb);
                 }
             }
         }
@@ -236,8 +242,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     const uint32_t *so = pk.symoff + (size_t)(f * 4 + q) * pk.Epad;
                     float *row = opnd + (size_t)(f * num_rot + q * nrr + i) * pk.Epad;
                     for (uint32_t e = threadIdx.x; e < pk.E; e += blockDim.x) {
-                        const uint32_t po = so[e];
-                        if ((po >> 24) == c) row[e] = sample_at(po & 0xffffffu);
+                        const uint32_t po = so[e], cc = (po >> 24) - c;      // (wraps below the block's first channel)
+                        if (cc < nch) row[e] = sample_at(cc * tile + (po & 0xffffffu));
                     }
                 }
         } else if constexpr (PACK >= 2) {
@@ -270,7 +276,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
 #pragma unroll
                 for (int w4 = 0; w4 < 4; ++w4) {
                     uint32_t p0, p1, p2, p3;
-                    if constexpr (use_lds) {
+                    if (!pk.wide) {
                         const uint2 pv = so4[w4];
                         p0 = pv.x & 0xffffu; p1 = pv.x >> 16; p2 = pv.y & 0xffffu; p3 = pv.y >> 16;
                     } else {
@@ -997,6 +1003,8 @@ struct pink_hip_ctx {
     bool trainer = false;
     bool use_lds = true;       // the rotation kernel keeps a block's base rotation in LDS
     bool image_lds = false;    // ... or, neurons too large for that, the image channel
+    uint32_t rot_nch = 1;      // channels per block of the rotation kernel: 1, or all of them (tiles side by side in LDS)
+    bool symoff_wide = false;  // byte-plane packing reads 32-bit table entries
     int device = 0;
     hipStream_t stream = nullptr;
 
@@ -1210,8 +1218,8 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
 {
     const bool store_variants = store != kStoreNone;
     Timed t(ctx, kClsRotate);
-    const dim3 grid(std::max(ctx->nrr, 1u), ctx->C, B);
-    const size_t lds = ctx->use_lds ? (size_t)ctx->D * ctx->Dp * sizeof(float)
+    const dim3 grid(std::max(ctx->nrr, 1u), ctx->C / ctx->rot_nch, B);
+    const size_t lds = ctx->use_lds ? (size_t)ctx->rot_nch * ctx->D * ctx->Dp * sizeof(float)
                      : ctx->image_lds ? (size_t)ctx->I * ctx->I * sizeof(float) : 0;
     // about four neuron pixels per thread: large neurons get large blocks, whose many waves per LDS
     // footprint hide the latency of the gathers (measured: 1024 threads 35 % faster than 256 at 3 x 70 x 70)
@@ -1226,6 +1234,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
         if (ctx->gemm) {
             pack = ctx->cfg.ed_type == PINK_HIP_UINT16 ? 3 : 2;
             pk.opnd = ctx->d_gPb; pk.norm = ctx->d_gnb; pk.rows_pad = ctx->Rp; pk.KS = ctx->gKS;
+            pk.wide = ctx->symoff_wide ? 1u : 0u;
         } else {
             pack = 1;
             pk.opnd = ctx->d_rotT; pk.rows_pad = ctx->Rpad;
@@ -1235,7 +1244,7 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
     hipLaunchKernelGGL((k_rotate<P_, L_>), grid, dim3(threads), lds, ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, \
                        ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D, ctx->cfg.num_rot, ctx->cfg.use_flip,               \
                        ctx->Dp, pk, store,                   \
-                       store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi)
+                       store_variants ? 0u : ctx->base_lo, store_variants ? ctx->D : ctx->base_hi, ctx->rot_nch)
 #define LAUNCH_ROTATE(P_)                         \
     do {                                          \
         if (ctx->use_lds) LAUNCH_ROTATE_(P_, 1);  \
@@ -1638,6 +1647,10 @@ int init_ctx(pink_hip_ctx *ctx)
     ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
     // the base rotation of a block lives in LDS: up to 158 of the CU's 160 KB (neurons up to 199 pixels wide)
     ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax;
+    // all channels of a base rotation in one block when their tiles fit together: multi-channel byte planes
+    // can then be packed by the rotation kernel (an operand piece may span two channels)
+    ctx->rot_nch = (ctx->use_lds && ctx->gemm && ctx->C > 1 && (size_t)ctx->C * ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax)
+                       ? ctx->C : 1u;
     ctx->image_lds = !ctx->use_lds && (size_t)ctx->I * ctx->I * sizeof(float) <= kRotateLdsMax;
     {
         const int lds = (int)kRotateLdsMax;          // per kernel, not per context: the most any context may ask
@@ -1653,7 +1666,7 @@ int init_ctx(pink_hip_ctx *ctx)
     // Operand packing inside the rotation kernel: float32 rows, or byte planes of single-channel
     // integer contexts, whenever the kernel keeps its base rotation in LDS.
     ctx->fused_pack = !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && (size_t)ctx->D * ctx->Dp < ((size_t)1 << 24) &&
-                      (ctx->gemm ? ctx->C == 1 : !is_int(ctx));
+                      (ctx->gemm ? (ctx->C == 1 || ctx->rot_nch == ctx->C) : !is_int(ctx));
     // Float variants of a whole launch group: for the update kernel and for a separate packing kernel.
     // The other contexts keep room for one image (pink_hip_rotate).
     ctx->pair_variants = ctx->trainer && ctx->fused_pack && ctx->S < (1u << 24);   // (the update kernel's divisions)
@@ -1755,14 +1768,17 @@ int init_ctx(pink_hip_ctx *ctx)
                 case 2: a = D - 1 - xs; bb = D - 1 - y; break;
                 default: a = y; bb = D - 1 - xs; break;
                 }
-                symoff[(size_t)sym * ctx->Epad + e] = (ch << 24) | (a * ctx->Dp + bb);     // LDS rows of Dp floats
+                // float rows: channel and position in the channel's tile (LDS rows of Dp floats); byte planes:
+                // position in the block's tiles, the channels' side by side
+                symoff[(size_t)sym * ctx->Epad + e] = ctx->gemm ? ch * D * ctx->Dp + a * ctx->Dp + bb : (ch << 24) | (a * ctx->Dp + bb);
                 ctx->base_lo = std::min({ctx->base_lo, a, bb});
                 ctx->base_hi = std::max({ctx->base_hi, a + 1, bb + 1});
             }
         }
         if (ctx->base_hi <= ctx->base_lo) ctx->base_lo = ctx->base_hi = 0;       // empty region
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
-        if (ctx->gemm && ctx->use_lds) {
+        ctx->symoff_wide = !(ctx->use_lds && (size_t)ctx->rot_nch * D * ctx->Dp <= 65536);
+        if (ctx->gemm && !ctx->symoff_wide) {
             // byte-plane packing out of an LDS tile reads 16-bit entries (single channel, positions below 40 000)
             std::vector<unsigned short> narrow(symoff.begin(), symoff.end());
             HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, narrow.data(), narrow.size() * sizeof(unsigned short), hipMemcpyHostToDevice));

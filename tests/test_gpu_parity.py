@@ -344,7 +344,7 @@ FUSED_TRAIN_SHAPES = [
     # N, C, I, D, nrot, flip, ed, shape, ed_type, images  -- operand packing inside the rotation and update kernels
     (10, 1, 20, 16, 24, True, 11, capi.CIRCULAR, capi.UINT16, 5),
     (70, 1, 20, 14, 8, False, 14, capi.QUADRATIC, capi.UINT8, 6),     # two column tiles, no flip
-    (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.UINT8, 4),        # three channels: packing stays in its own kernel
+    (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.UINT8, 4),        # three channels: their base rotations side by side in LDS, byte planes packed by the rotation kernel
     (6, 3, 12, 10, 8, True, 6, capi.QUADRATIC, capi.FLOAT, 4),        # three channels, float32 rows from the rotation kernel
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.FLOAT, 3),           # region repeats channel 0 (CPU rule): no inverse table
     (5, 2, 9, 8, 4, True, 7, capi.CIRCULAR, capi.UINT16, 3),
