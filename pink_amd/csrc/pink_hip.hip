@@ -1492,8 +1492,8 @@ int init_ctx(pink_hip_ctx *ctx)
                                               "whose packed SOM fits in LDS");
         ctx->mfma = fits && (c.kernel_choice == PINK_HIP_KERNEL_AUTO || c.kernel_choice == PINK_HIP_KERNEL_MFMA);
     }
-    // Symmetries on the SOM side: needs the union of the symmetric images of the region to fit 32
-    // k-steps held in registers and at most 96 base rotations per image.
+    // Symmetries on the SOM side: needs the union of the symmetric images of the region to fit 64
+    // k-steps held in registers and at most 256 base rotations per image (8 row tiles).
     {
         const uint32_t D = ctx->D, DD = D * D;
         std::vector<std::vector<uint32_t>> pos(8);      // pos[sym][e] = perm_sym(region[e])
@@ -1539,11 +1539,11 @@ int init_ctx(pink_hip_ctx *ctx)
             for (uint32_t e = 0; e < ctx->E; ++e) { if (seen[region[e]]) distinct = false; seen[region[e]] = 1; }
         }
         const size_t lds_img = pink_sym::lds_image_bytes(ctx->C, ctx->I);
-        const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 64 && ctx->RTP <= 3 &&
+        const bool fits_sym = c.ed_type == PINK_HIP_UINT8 && !ctx->trainer && distinct && ks_need <= 64 && ctx->RTP <= 8 &&
                               lds_img <= 150 * 1024 && D < 4096 && ctx->C < 256;
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM && !fits_sym)
             return fail(ctx, PINK_HIP_EINVAL, "the symmetric MFMA distance kernel needs a uint8 mapper, at most 2048 "
-                                              "region elements (union over the symmetries) and at most 384 rotations");
+                                              "region elements (union over the symmetries) and at most 1024 rotations");
         ctx->mfma_sym = fits_sym && (c.kernel_choice == PINK_HIP_KERNEL_AUTO || c.kernel_choice == PINK_HIP_KERNEL_MFMA_SYM);
         if (ctx->mfma_sym) {
             ctx->mfma = false;

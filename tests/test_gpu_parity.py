@@ -70,6 +70,8 @@ DIST_SHAPES = [
     (5, 1, 8, 8, 1, True, 5, capi.QUADRATIC),
     (331, 1, 150, 106, 360, True, 75, capi.CIRCULAR),     # cfg 2
     (1600, 3, 100, 70, 180, True, 50, capi.QUADRATIC),    # cfg 3
+    (7, 1, 40, 28, 720, True, 20, capi.QUADRATIC),        # 1440 variants: six row tiles of base rotations
+    (3, 1, 30, 20, 1024, False, 15, capi.CIRCULAR),       # eight
     (5, 1, 160, 226, 8, True, 113, capi.QUADRATIC),       # neurons too large for an LDS tile: the image in LDS
     (5, 1, 290, 205, 8, True, 40, capi.CIRCULAR),         # ... nothing in LDS
     (5, 1, 128, 181, 16, True, 90, capi.QUADRATIC),       # a 128 KiB base rotation in LDS
