@@ -146,7 +146,6 @@ struct PackArgs {
     void *opnd;            // float rows, or byte planes
     long long *norm;       // integer modes: [b][Rp]
     uint32_t E, Epad, rows_pad, KS;
-    uint32_t wide;         // integer modes: table entries of 32 bits (else 16)
 };
 
 template <int PACK, int TILE>
@@ -218,23 +217,24 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         // 1: all; 2: the base rotation and its quarter turn, of which the other six are row and column
         // reversals (the update kernel reads them that way)
         const uint32_t nf_st = store_variants == 2 ? 1u : nf, nq_st = store_variants == 2 ? min(nq, 2u) : nq;
-        for (uint32_t p = threadIdx.x; p < (store_variants ? DD : 0u); p += blockDim.x) {
-            const uint32_t x = p / D, y = p % D;
-            for (uint32_t f = 0; f < nf_st; ++f) {
-                const uint32_t xs = f ? D - 1 - x : x;
-                for (uint32_t q = 0; q < nq_st; ++q) {
-                    uint32_t a, bb;
-                    switch (q) {
-                    case 0: a = xs; bb = y; break;
-                    case 1: a = D - 1 - y; bb = xs; break;
-                    case 2: a = D - 1 - xs; bb = D - 1 - y; break;
-                    default: a = y; bb = D - 1 - xs; break;
+        for (uint32_t cc = 0; cc < (store_variants ? nch : 0u); ++cc)
+            for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
+                const uint32_t x = p / D, y = p % D;
+                for (uint32_t f = 0; f < nf_st; ++f) {
+                    const uint32_t xs = f ? D - 1 - x : x;
+                    for (uint32_t q = 0; q < nq_st; ++q) {
+                        uint32_t a, bb;
+                        switch (q) {
+                        case 0: a = xs; bb = y; break;
+                        case 1: a = D - 1 - y; bb = xs; break;
+                        case 2: a = D - 1 - xs; bb = D - 1 - y; break;
+                        default: a = y; bb = D - 1 - xs; break;
+                        }
+                        const uint32_t k = f * num_rot + q * nrr + i;
+                        out[((size_t)k * C + c + cc) * DD + p] = sample(cc, a, bb);
                     }
-                    const uint32_t k = f * num_rot + q * nrr + i;
-                    for (uint32_t cc = 0; cc < nch; ++cc) out[((size_t)k * C + c + cc) * DD + p] = sample(cc, a, bb);
                 }
             }
-        }
         if constexpr (PACK == 1) {
             float *opnd = (float *)pk.opnd + (size_t)b * pk.rows_pad * pk.Epad;
             for (uint32_t f = 0; f < nf; ++f)
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                 const uint32_t si = item % nsym, piece = item / nsym;   // neighbouring lanes: the adjacent rows of one piece
                 const uint32_t f = si / nq, q = si % nq, sym = f * 4 + q;
                 const uint32_t r = i * nsym + si;             // operand row: the symmetries of a base rotation are adjacent
-                // (16-bit table entries with an LDS tile: one channel, at most 40 000 floats; 32-bit without)
+                // (16-bit table entries with LDS tiles: at most 40 448 floats; 32-bit without)
                 const uint2 *so4 = (const uint2 *)((const unsigned short *)pk.symoff + (size_t)sym * pk.Epad + piece * 16);
                 const uint4 *so4w = (const uint4 *)(pk.symoff + (size_t)sym * pk.Epad + piece * 16);
                 v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
 #pragma unroll
                 for (int w4 = 0; w4 < 4; ++w4) {
                     uint32_t p0, p1, p2, p3;
-                    if (!pk.wide) {
+                    if constexpr (use_lds) {
                         const uint2 pv = so4[w4];
                         p0 = pv.x & 0xffffu; p1 = pv.x >> 16; p2 = pv.y & 0xffffu; p3 = pv.y >> 16;
                     } else {
@@ -1004,7 +1004,6 @@ struct pink_hip_ctx {
     bool use_lds = true;       // the rotation kernel keeps a block's base rotation in LDS
     bool image_lds = false;    // ... or, neurons too large for that, the image channel
     uint32_t rot_nch = 1;      // channels per block of the rotation kernel: 1, or all of them (tiles side by side in LDS)
-    bool symoff_wide = false;  // byte-plane packing reads 32-bit table entries
     int device = 0;
     hipStream_t stream = nullptr;
 
@@ -1234,7 +1233,6 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
         if (ctx->gemm) {
             pack = ctx->cfg.ed_type == PINK_HIP_UINT16 ? 3 : 2;
             pk.opnd = ctx->d_gPb; pk.norm = ctx->d_gnb; pk.rows_pad = ctx->Rp; pk.KS = ctx->gKS;
-            pk.wide = ctx->symoff_wide ? 1u : 0u;
         } else {
             pack = 1;
             pk.opnd = ctx->d_rotT; pk.rows_pad = ctx->Rpad;
@@ -1628,17 +1626,14 @@ int init_ctx(pink_hip_ctx *ctx)
             ctx->Np = round_up(ctx->N, 64);
             ctx->Rp = round_up(ctx->R, 64);
             const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
-            // k is cut into as many slices as keep all blocks (one per tile and slice, four waves each)
-            // resident at once, one per CU, with at least four k-steps per wave (measured at 72 tiles:
-            // 3 slices = 216 blocks beat 2 by 4 % and 4, a second round of blocks, by 30 %)
-            uint32_t slices = std::max(1u, (uint32_t)ctx->num_cu / tiles);
-            slices = std::min(slices, std::max(1u, ctx->gKS / 16));
-            // Cutting k costs a second launch (about 5 us, the time of some 300 MFMAs): with fewer than 256
-            // MFMAs per wave one block per tile is faster, which then finishes the tile itself (measured at
-            // 64 k-steps: uint8, 64 MFMAs per wave, 47 k images/s in one slice against 43 k in four; uint16,
-            // 256 per wave, the break-even)
-            const uint32_t mfma_per_wave = ((ctx->gKS + 3) / 4) * (c.ed_type == PINK_HIP_UINT16 ? 16u : 4u);
-            if (mfma_per_wave < 256) slices = 1;
+            // k is cut into slices (blocks per tile, four waves each) so that a wave has about 16 k-steps
+            // (uint8: 64 MFMAs) or 11 (uint16: 176), never more blocks than CUs.  Cutting costs a second
+            // launch that adds the slices up; one slice finishes its tile itself.  Measured optima, images/s
+            // against one slice: 12 tiles x 235 k-steps uint8: 4 slices, +21 %; 24 x 254 uint8: 4, +15 %;
+            // 24 x 254 uint16: 6, +37 %; 72 x 135 uint16: 3; 24 x 64 uint8 and 84 x 141 uint8: 1.
+            const uint32_t per_wave = c.ed_type == PINK_HIP_UINT16 ? 11u : 16u;
+            uint32_t slices = (ctx->gKS + 4 * per_wave - 1) / (4 * per_wave);
+            slices = std::max(1u, std::min(slices, (uint32_t)ctx->num_cu / tiles));
             ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
             ctx->gslices = (ctx->gKS + 4 * ctx->gks_per - 1) / (4 * ctx->gks_per);
         }
@@ -1777,8 +1772,7 @@ int init_ctx(pink_hip_ctx *ctx)
         }
         if (ctx->base_hi <= ctx->base_lo) ctx->base_lo = ctx->base_hi = 0;       // empty region
         TRY(dev_alloc(ctx, &ctx->d_symoff, symoff.size()));
-        ctx->symoff_wide = !(ctx->use_lds && (size_t)ctx->rot_nch * D * ctx->Dp <= 65536);
-        if (ctx->gemm && !ctx->symoff_wide) {
+        if (ctx->gemm && ctx->use_lds) {        // (an LDS tile set has at most 40 448 floats)
             // byte-plane packing out of an LDS tile reads 16-bit entries (single channel, positions below 40 000)
             std::vector<unsigned short> narrow(symoff.begin(), symoff.end());
             HIP_TRY(ctx, hipMemcpy(ctx->d_symoff, narrow.data(), narrow.size() * sizeof(unsigned short), hipMemcpyHostToDevice));
