@@ -1001,6 +1001,7 @@ struct pink_hip_ctx {
     uint32_t shift = 32;       // key = value << shift | rotation
     uint32_t factor = 1;       // 255 / 65535 in the integer modes
     bool trainer = false;
+    bool wide_sums = false;    // integer sums need more than 31 bits
     bool use_lds = true;       // the rotation kernel keeps a block's base rotation in LDS
     bool image_lds = false;    // ... or, neurons too large for that, the image channel
     uint32_t rot_nch = 1;      // channels per block of the rotation kernel: 1, or all of them (tiles side by side in LDS)
@@ -1376,7 +1377,10 @@ int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     if (!ctx->d_somP || !ctx->d_rotT) return fail(ctx, PINK_HIP_ESTATE, "distance operands were not allocated");
     switch (ctx->cfg.ed_type) {
     case PINK_HIP_FLOAT: launch_dist_f32(ctx, slot, B); break;
-    case PINK_HIP_UINT8: launch_dist<1>(ctx, slot, B); break;
+    case PINK_HIP_UINT8:
+        if (ctx->wide_sums) launch_dist<2>(ctx, slot, B);
+        else launch_dist<1>(ctx, slot, B);
+        break;
     default: launch_dist<2>(ctx, slot, B); break;
     }
     return launch_check(ctx, "k_dist");
@@ -1464,8 +1468,9 @@ int init_ctx(pink_hip_ctx *ctx)
     if (is_int(ctx)) {
         // key = ssd << 16 | rotation: the sum must stay below 2^48 and R below 2^16.
         const double max_ssd = (double)ctx->factor * ctx->factor * ctx->E;
-        if (ctx->R > 65536 || max_ssd >= 281474976710656.0 || (c.ed_type == PINK_HIP_UINT8 && max_ssd >= 2147483648.0))
+        if (ctx->R > 65536 || max_ssd >= 281474976710656.0)
             return fail(ctx, PINK_HIP_EINVAL, "distance region or rotation count too large for the integer distance modes");
+        ctx->wide_sums = max_ssd >= 2147483648.0;          // uint8 beyond 33 025 elements: 64-bit sums like uint16
     }
     TRY(dev_alloc(ctx, &ctx->d_region, region.size()));
     HIP_TRY(ctx, hipMemcpy(ctx->d_region, region.data(), region.size() * sizeof(uint32_t), hipMemcpyHostToDevice));

@@ -357,6 +357,8 @@ FUSED_TRAIN_SHAPES = [
     (4, 1, 160, 226, 8, True, 113, capi.QUADRATIC, capi.UINT8, 2),    # ... but the image fits: interpolated out of LDS
     (3, 1, 160, 226, 8, True, 113, capi.CIRCULAR, capi.UINT16, 2),
     (3, 1, 150, 201, 8, True, 100, capi.QUADRATIC, capi.FLOAT, 2),
+    (3, 1, 150, 200, 4, True, 200, capi.QUADRATIC, capi.UINT8, 2),    # 40 000 region elements: uint8 sums beyond 31 bits
+    (2, 1, 150, 200, 4, False, 190, capi.QUADRATIC, capi.UINT16, 2),  # ... and uint16 beyond the matrix-core path's row length
     (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
 ]
 
