@@ -1621,12 +1621,17 @@ int init_ctx(pink_hip_ctx *ctx)
     // problems pad their rows to one 64 x 64 tile; they are latency bound either way and the four
     // waves of a block still cut k four ways.
     {
-        const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->Epad <= 32768;   // planes of a row fit LDS
+        // the byte planes of a row are staged in LDS when a row is packed by a kernel of its own (128 KB), and the
+        // uint16 accumulator that takes two byte products per element stays exact in int32 for 65 535 elements
+        const bool applies = is_int(ctx) && !ctx->mfma && !ctx->mfma_sym && ctx->Epad < 65536;
         if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM && !applies)
             return fail(ctx, PINK_HIP_EINVAL, "the MFMA GEMM distance kernel needs an integer distance type");
         ctx->gemm = applies && (c.kernel_choice == PINK_HIP_KERNEL_MFMA_GEMM ||
                                 c.kernel_choice == PINK_HIP_KERNEL_AUTO);
         if (ctx->gemm) {
+            // (limits are per kernel, not per context)
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_pack_planes<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 65536));
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_pack_planes<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
             ctx->gKS = ctx->Epad / 32;
             ctx->Np = round_up(ctx->N, 64);
             ctx->Rp = round_up(ctx->R, 64);

@@ -358,7 +358,9 @@ FUSED_TRAIN_SHAPES = [
     (3, 1, 160, 226, 8, True, 113, capi.CIRCULAR, capi.UINT16, 2),
     (3, 1, 150, 201, 8, True, 100, capi.QUADRATIC, capi.FLOAT, 2),
     (3, 1, 150, 200, 4, True, 200, capi.QUADRATIC, capi.UINT8, 2),    # 40 000 region elements: uint8 sums beyond 31 bits
-    (2, 1, 150, 200, 4, False, 190, capi.QUADRATIC, capi.UINT16, 2),  # ... and uint16 beyond the matrix-core path's row length
+    (2, 1, 150, 200, 4, False, 190, capi.QUADRATIC, capi.UINT16, 2),
+    (2, 1, 100, 257, 4, False, 257, capi.QUADRATIC, capi.UINT8, 2),   # 66 049: beyond the matrix-core path's row length
+    (2, 1, 100, 256, 4, False, 256, capi.QUADRATIC, capi.UINT16, 2),  # 65 536 (uint16 sums reach 2^48 just above that)
     (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
 ]
 
@@ -432,6 +434,23 @@ def test_contexts_of_different_sizes_side_by_side():
     finally:
         for m in made:
             m[0].close()
+
+
+@pytest.mark.parametrize("ed_type,factor", [(capi.UINT8, 255), (capi.UINT16, 65535)])
+def test_largest_matrix_core_region_with_extreme_data(ed_type, factor):
+    # 65 025 region elements, all of them at one end of the range in both operands: the byte-plane dot
+    # products are as large as they get (closed form: 0, and factor^2 * elements)
+    say("largest region on the matrix cores", ed_type)
+    D = 255
+    som = np.zeros((2, D * D), np.float32)
+    som[1] = 1.0
+    with capi.Context(2, 1, D, D, 1, False, D, capi.QUADRATIC, ed_type) as ctx:
+        assert ctx.distance_kernel == capi.KERNEL_MFMA_GEMM
+        ctx.set_som(som)
+        for value in (0.0, 1.0):
+            d, ssd, best = ctx.distance(np.full((1, D, D), value, np.float32))
+            want = [0, factor * factor * D * D] if value == 0.0 else [factor * factor * D * D, 0]
+            assert ssd.tolist() == want and best.tolist() == [0, 0]
 
 
 def test_reference_mapper_known_answers():
