@@ -48,6 +48,20 @@ def test_rotate_bit_exact(C_, I, D, nrot, flip):
     assert np.array_equal(bits(got), bits(want))
 
 
+@pytest.mark.parametrize("ed_type", [capi.UINT8, capi.UINT16])
+def test_rotate_tap_on_integer_contexts_with_channels(ed_type):
+    # integer contexts keep the base rotations of all channels in one block of the rotation kernel
+    C_, I, D, nrot, flip = 3, 20, 14, 8, True
+    say("rotate tap, integer, channels", ed_type)
+    rng = np.random.default_rng(ed_type)
+    img = rng.random((C_, I, I), dtype=np.float32)
+    want = O.rotated_images(img, C_, I, D, nrot, flip)
+    F = capi.make_update_factors(capi.CARTESIAN, [3], capi.GAUSSIAN, 1.0, 0.5)
+    for factors in (None, F):
+        with capi.Context(3, C_, I, D, nrot, flip, 9, capi.QUADRATIC, ed_type, factors) as ctx:
+            assert np.array_equal(bits(ctx.rotate(img)), bits(want))
+
+
 def test_rotate_reference_golden():
     # test/SelfOrganizingMapTest/generate_rotated_images.cpp:15-41
     with capi.Context(1, 1, 2, 2, 4, False, 2) as ctx:
