@@ -317,6 +317,25 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     }
 }
 
+// Where a packing kernel finds variant r when only two of a base rotation's eight symmetries are
+// stored (the base rotation and its quarter turn): the stored variant to read and the region offsets
+// to read it with -- the region under the row and/or column reversal that turns the stored variant
+// into variant r (see k_update).  off4 = null: every variant is stored, `off` is used as it is.
+struct PairSource {
+    const uint32_t *off4;      // [rows reversed * 2 + columns reversed][E]
+    uint32_t num_rot, nrr, E;
+};
+
+__device__ __forceinline__ void pair_source(const PairSource &ps, uint32_t r, uint32_t &src, const uint32_t *&off)
+{
+    src = r;
+    if (!ps.off4) return;
+    const uint32_t f = r >= ps.num_rot ? 1u : 0u, rem = r - f * ps.num_rot;
+    const uint32_t q = rem / ps.nrr, i = rem - q * ps.nrr;
+    src = (q & 1) * ps.nrr + i;
+    off = ps.off4 + (size_t)((f ^ (q >> 1)) * 2 + (q >> 1)) * ps.E;
+}
+
 // ---------------------------------------------------------------------------------
 // Operand packing for the vector-ALU distance kernels.
 //   somP[n][k]    = conv(som[n][off[k]])                      k < E, 0 beyond (row length Epad)
@@ -343,7 +362,7 @@ __global__ __launch_bounds__(256) void k_pack_som(const float *__restrict__ som,
 template <bool QUANT>
 __global__ __launch_bounds__(256) void k_pack_rot(const float *__restrict__ rot, const uint32_t *__restrict__ off,
                                                   void *__restrict__ rotT, uint32_t R, uint32_t S, uint32_t E,
-                                                  uint32_t Epad, uint32_t Rpad, float factor)
+                                                  uint32_t Epad, uint32_t Rpad, float factor, PairSource ps)
 {
     __shared__ float tile[32][33];
     const uint32_t b = blockIdx.z;
@@ -351,7 +370,10 @@ __global__ __launch_bounds__(256) void k_pack_rot(const float *__restrict__ rot,
     const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
     for (uint32_t rr = ty; rr < 32; rr += 8) {
         const uint32_t r = r0 + rr, k = k0 + tx;
-        tile[rr][tx] = (r < R && k < E) ? rot[((size_t)b * R + r) * S + off[k]] : 0.0f;
+        uint32_t src = r;
+        const uint32_t *o = off;
+        if (r < R) pair_source(ps, r, src, o);
+        tile[rr][tx] = (r < R && k < E) ? rot[((size_t)b * R + src) * S + o[k]] : 0.0f;
     }
     __syncthreads();
     for (uint32_t kk = ty; kk < 32; kk += 8) {
@@ -367,13 +389,18 @@ __global__ __launch_bounds__(256) void k_pack_rot(const float *__restrict__ rot,
 // every variant contiguous in k (rows r >= R and elements k >= E are zero).
 __global__ __launch_bounds__(256) void k_pack_rot_rows(const float *__restrict__ rot, const uint32_t *__restrict__ off,
                                                        float *__restrict__ rotP, uint32_t R, uint32_t S, uint32_t E,
-                                                       uint32_t Epad, uint32_t Rpad)
+                                                       uint32_t Epad, uint32_t Rpad, PairSource ps)
 {
     const uint32_t b = blockIdx.z, r = blockIdx.y;
     const uint32_t k = blockIdx.x * 256 + threadIdx.x;
     if (k >= Epad) return;
     float v = 0.0f;
-    if (r < R && k < E) v = rot[((size_t)b * R + r) * S + off[k]];
+    if (r < R && k < E) {
+        uint32_t src;
+        const uint32_t *o = off;
+        pair_source(ps, r, src, o);
+        v = rot[((size_t)b * R + src) * S + o[k]];
+    }
     rotP[((size_t)b * Rpad + r) * Epad + k] = v;
 }
 
@@ -1040,6 +1067,8 @@ struct pink_hip_ctx {
     uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
+    bool pair_pack = false;                // no LDS tile of any kind: two symmetries stored, the packing kernels read the rest out of them
+    uint32_t *d_region4 = nullptr;         // the region under the four row/column reversals (pair_pack)
     bool pair_variants = false;            // trainer: k_rotate stores two of the eight symmetries of a base rotation
     bool fused_som = false;                // integer GEMM trainer: k_update refreshes the SOM planes and norms itself
     uint32_t na_cur = 0;                   // which half of d_gna holds the norms of the current SOM operand
@@ -1186,10 +1215,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
             hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(1024), 2 * ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
         else
             hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(1024), ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr);
+                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
         return launch_check(ctx, "k_pack_planes");
     }
     if (ctx->mfma_sym) {
@@ -1265,27 +1294,31 @@ int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 {
     if (ctx->fused_pack) return PINK_HIP_OK;              // k_rotate wrote the operand already
     Timed t(ctx, kClsPack);
+    PairSource ps{};
+    if (ctx->pair_pack) { ps.off4 = ctx->d_region4; ps.num_rot = ctx->cfg.num_rot; ps.nrr = std::max(ctx->nrr, 1u); ps.E = ctx->E; }
     if (ctx->gemm) {
+        // long rows: large blocks, so that a CU (a few blocks by their LDS rows) still runs all its waves
+        const uint32_t pack_threads = ctx->gKS * 32 >= 4096 ? 1024 : 256;
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
-            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(256), 2 * ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
-                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow);
+            hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->R, B), dim3(pack_threads), 2 * ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow, ps);
         else
-            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(256), ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
-                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow);
+            hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->R, B), dim3(pack_threads), ctx->gKS * 32, ctx->stream, ctx->d_rot, ctx->d_region,
+                               ctx->d_gPb, ctx->d_gnb, ctx->R, ctx->Rp, ctx->S, ctx->E, ctx->gKS, ctx->d_grow, ps);
         return launch_check(ctx, "k_pack_planes");
     }
     if (!is_int(ctx)) {
         hipLaunchKernelGGL(k_pack_rot_rows, dim3((ctx->Epad + 255) / 256, ctx->Rpad, B), dim3(256), 0, ctx->stream,
-                           ctx->d_rot, ctx->d_region, (float *)ctx->d_rotT, ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad);
+                           ctx->d_rot, ctx->d_region, (float *)ctx->d_rotT, ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, ps);
         return launch_check(ctx, "k_pack_rot_rows");
     }
     const dim3 grid(ctx->Epad / 32, ctx->Rpad / 32, B);
     if (is_int(ctx))
         hipLaunchKernelGGL(k_pack_rot<true>, grid, dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region, ctx->d_rotT,
-                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, (float)ctx->factor);
+                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, (float)ctx->factor, ps);
     else
         hipLaunchKernelGGL(k_pack_rot<false>, grid, dim3(256), 0, ctx->stream, ctx->d_rot, ctx->d_region, ctx->d_rotT,
-                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, 1.0f);
+                           ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, 1.0f, ps);
     return launch_check(ctx, "k_pack_rot");
 }
 
@@ -1428,7 +1461,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
@@ -1672,9 +1705,25 @@ int init_ctx(pink_hip_ctx *ctx)
     // integer contexts, whenever the kernel keeps its base rotation in LDS.
     ctx->fused_pack = !ctx->mfma && !ctx->mfma_sym && ctx->C < 256 && (size_t)ctx->D * ctx->Dp < ((size_t)1 << 24) &&
                       (ctx->gemm ? (ctx->C == 1 || ctx->rot_nch == ctx->C) : !is_int(ctx));
+    // Neither the base rotation nor the image fits LDS: interpolating every packed element out of global
+    // memory is slow, so the rotation kernel stores two symmetries and packing kernels of their own read
+    // all eight out of those, with coalesced accesses
+    ctx->pair_pack = !ctx->use_lds && !ctx->image_lds && !ctx->mfma && !ctx->mfma_sym && ctx->S < (1u << 24);
+    if (ctx->pair_pack) {
+        ctx->fused_pack = false;
+        const uint32_t D = ctx->D, DD = D * D;
+        std::vector<uint32_t> region4((size_t)4 * ctx->E);
+        for (uint32_t combo = 0; combo < 4; ++combo)
+            for (uint32_t k = 0; k < ctx->E; ++k) {
+                const uint32_t ch = region[k] / DD, x = (region[k] % DD) / D, y = region[k] % D;
+                region4[(size_t)combo * ctx->E + k] = ch * DD + ((combo >> 1) ? D - 1 - x : x) * D + ((combo & 1) ? D - 1 - y : y);
+            }
+        TRY(dev_alloc(ctx, &ctx->d_region4, region4.size()));
+        HIP_TRY(ctx, hipMemcpy(ctx->d_region4, region4.data(), region4.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+    }
     // Float variants of a whole launch group: for the update kernel and for a separate packing kernel.
     // The other contexts keep room for one image (pink_hip_rotate).
-    ctx->pair_variants = ctx->trainer && ctx->fused_pack && ctx->S < (1u << 24);   // (the update kernel's divisions)
+    ctx->pair_variants = ctx->trainer && (ctx->fused_pack || ctx->pair_pack) && ctx->S < (1u << 24);   // (the update kernel's divisions)
     const bool group_variants = ctx->trainer || !(ctx->mfma || ctx->mfma_sym || ctx->fused_pack);
 
     // Launch-group size: one image for a trainer; for a mapper as many as fit ~4 GiB.
@@ -1885,7 +1934,7 @@ int distance_group(pink_hip_ctx *ctx, const float *dev_images, uint32_t B)
         return PINK_HIP_OK;
     }
     // the variants themselves are only read by the update kernel and by a separate packing kernel
-    TRY(run_rotate(ctx, dev_images, B, ctx->fused_pack ? kStoreNone : kStoreAll));
+    TRY(run_rotate(ctx, dev_images, B, ctx->fused_pack ? kStoreNone : ctx->pair_pack ? kStorePair : kStoreAll));
     TRY(run_pack_rot(ctx, B));
     TRY(run_dist(ctx, 0, B));
     return PINK_HIP_OK;
