@@ -317,6 +317,104 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     }
 }
 
+// The base rotation and its quarter turn for images and neurons of any size (neither fits LDS): a
+// block computes one 32 x 32 tile of base rotation i of one channel.  The pixels of the image that
+// the tile's interpolations touch lie in a window of at most 50 x 50 (the tile turned by up to 90
+// degrees, plus the neighbours), which goes to LDS first; the arithmetic is base_pixel's, tap by tap.
+// The tile is written twice, row-major both times: as it is into variant i, and turned,
+// Q1[x][y] = B[D-1-y][x], into variant nrr + i (through LDS, so that both stores run along rows).
+// A sample whose neighbours the window does not hold (on the last row or column of the image, where
+// base_pixel's clamped neighbour index leaves the row) is left to base_pixel itself.
+constexpr uint32_t kRotTile = 32, kRotWindow = 52;
+
+__global__ __launch_bounds__(256) void k_rotate_pair_tiled(const float *__restrict__ images, float *__restrict__ rot,
+                                                           const float *__restrict__ cos_t, const float *__restrict__ sin_t,
+                                                           unsigned long long *__restrict__ key, uint32_t N, uint32_t C,
+                                                           uint32_t I, uint32_t D, uint32_t num_rot, uint32_t use_flip,
+                                                           uint32_t tiles_per_row)
+{
+    __shared__ float s_win[kRotWindow * kRotWindow];
+    __shared__ float s_out[kRotTile][kRotTile + 1];
+    const uint32_t tile = blockIdx.x, i = blockIdx.y, c = blockIdx.z % C, b = blockIdx.z / C;
+    const uint32_t a0 = (tile / tiles_per_row) * kRotTile, b0 = (tile % tiles_per_row) * kRotTile;
+    const uint32_t nrr = num_rot / 4, R = num_rot * (use_flip ? 2u : 1u), DD = D * D;
+    const float *img = images + ((size_t)b * C + c) * I * I;
+    float *out = rot + (size_t)b * R * C * DD;
+    const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
+    const uint32_t tid = threadIdx.x;
+    if (tile == 0 && i == 0 && c == 0)
+        for (uint32_t n = tid; n < N; n += blockDim.x) key[(size_t)b * N + n] = ~0ull;
+
+    const uint32_t a1 = min(a0 + kRotTile, D), b1 = min(b0 + kRotTile, D);        // the tile: rows [a0, a1), columns [b0, b1)
+    // source window [wx0, wx1] x [wy0, wy1] of the tile's corners, one pixel of margin on every side
+    const float src_c = __fmul_rn((float)(I - 1), 0.5f), dst_c = __fmul_rn((float)(D - 1), 0.5f);
+    int wx0 = 0, wx1 = -1, wy0 = 0, wy1 = -1;
+    if (i) {
+        float lo_x = 3.0e38f, hi_x = -3.0e38f, lo_y = 3.0e38f, hi_y = -3.0e38f;
+#pragma unroll
+        for (int corner = 0; corner < 4; ++corner) {
+            const float px = __fsub_rn((float)((corner & 1) ? a1 - 1 : a0), dst_c);
+            const float py = __fsub_rn((float)((corner & 2) ? b1 - 1 : b0), dst_c);
+            const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+            const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+            lo_x = fminf(lo_x, sxf); hi_x = fmaxf(hi_x, sxf); lo_y = fminf(lo_y, syf); hi_y = fmaxf(hi_y, syf);
+        }
+        wx0 = max(0, (int)floorf(lo_x) - 1); wx1 = min((int)I - 1, (int)floorf(hi_x) + 2);
+        wy0 = max(0, (int)floorf(lo_y) - 1); wy1 = min((int)I - 1, (int)floorf(hi_y) + 2);
+        // a tile that maps beyond the image (neurons larger than the image) has an empty window: every
+        // sample is then outside; a window beyond the LDS array cannot occur, and would send all samples
+        // down the slow path
+        if (wx1 < wx0 || wy1 < wy0 || wx1 - wx0 + 1 > (int)kRotWindow || wy1 - wy0 + 1 > (int)kRotWindow) { wx1 = wx0 - 1; wy1 = wy0 - 1; }
+    }
+    const int ww = wy1 - wy0 + 1, wh = wx1 - wx0 + 1;
+    for (int p = (int)tid; p < ww * wh; p += (int)blockDim.x) {
+        const int r = p / ww, q = p - r * ww;
+        s_win[r * ww + q] = img[(size_t)(wx0 + r) * I + (wy0 + q)];
+    }
+    __syncthreads();
+
+    const uint32_t tx = tid & 31, ty = tid >> 5;
+    for (uint32_t rr = ty; rr < kRotTile; rr += 8) {
+        const uint32_t x = a0 + rr, y = b0 + tx;
+        float v = 0.0f;
+        if (x < D && y < D) {
+            bool done = false;
+            if (i) {
+                const float px = __fsub_rn((float)x, dst_c), py = __fsub_rn((float)y, dst_c);
+                const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+                const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+                const float lim = (float)(I - 1);
+                if (sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim) {
+                    done = true;                           // outside the image: 0
+                } else {
+                    const int ix = (int)sxf, iy = (int)syf;
+                    if (ix >= wx0 && ix + 1 <= wx1 && iy >= wy0 && iy + 1 <= wy1) {
+                        const float rx = __fsub_rn(sxf, (float)ix), ry = __fsub_rn(syf, (float)iy);
+                        const float cx = __fsub_rn(1.0f, rx), cy = __fsub_rn(1.0f, ry);
+                        const float *t = s_win + (ix - wx0) * ww + (iy - wy0);
+                        const float ta = __fmul_rn(__fmul_rn(cx, cy), t[0]);
+                        const float tb = __fmul_rn(__fmul_rn(cx, ry), t[1]);
+                        const float tc = __fmul_rn(__fmul_rn(rx, cy), t[ww]);
+                        const float td = __fmul_rn(__fmul_rn(rx, ry), t[ww + 1]);
+                        v = __fadd_rn(__fadd_rn(__fadd_rn(ta, tb), tc), td);
+                        done = true;
+                    }
+                }
+            }
+            if (!done) v = base_pixel(img, I, D, i, cs, sn, x, y);
+            out[((size_t)i * C + c) * DD + (size_t)x * D + y] = v;
+        }
+        s_out[rr][tx] = v;
+    }
+    if (num_rot == 1) return;                               // a single rotation has no quarter turns
+    __syncthreads();
+    // Q1[x][y] = B[D-1-y][x]: row x = b0 + r of Q1 takes column r of the tile, rows a1-1 down to a0
+    for (uint32_t r = ty; r < kRotTile; r += 8) {
+        const uint32_t x = b0 + r, aa = a1 - 1 - tx;         // tile row read by this lane (wraps below a0)
+        if (x < D && tx < a1 - a0) out[((size_t)(nrr + i) * C + c) * DD + (size_t)x * D + (D - 1 - aa)] = s_out[aa - a0][r];
+    }
+}
+
 // Where a packing kernel finds variant r when only two of a base rotation's eight symmetries are
 // stored (the base rotation and its quarter turn): the stored variant to read and the region offsets
 // to read it with -- the region under the row and/or column reversal that turns the stored variant
@@ -1247,6 +1345,13 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
 {
     const bool store_variants = store != kStoreNone;
     Timed t(ctx, kClsRotate);
+    if (ctx->pair_pack && store == kStorePair) {
+        const uint32_t tiles_per_row = (ctx->D + kRotTile - 1) / kRotTile;
+        hipLaunchKernelGGL(k_rotate_pair_tiled, dim3(tiles_per_row * tiles_per_row, std::max(ctx->nrr, 1u), ctx->C * B), dim3(256), 0,
+                           ctx->stream, dev_images, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_key, ctx->N, ctx->C, ctx->I, ctx->D,
+                           ctx->cfg.num_rot, ctx->cfg.use_flip, tiles_per_row);
+        return launch_check(ctx, "k_rotate_pair_tiled");
+    }
     const dim3 grid(std::max(ctx->nrr, 1u), ctx->C / ctx->rot_nch, B);
     const size_t lds = ctx->use_lds ? (size_t)ctx->rot_nch * ctx->D * ctx->Dp * sizeof(float)
                      : ctx->image_lds ? (size_t)ctx->I * ctx->I * sizeof(float) : 0;

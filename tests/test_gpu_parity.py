@@ -34,6 +34,7 @@ ROT_SHAPES = [
     (1, 290, 205, 8, True),     # 205*205*4 B > 158 KiB and so is the image: nothing in LDS
     (1, 150, 205, 16, True),    # the image in LDS instead of the base rotation
     (2, 160, 226, 8, False),
+    (1, 210, 260, 8, True),     # nothing in LDS, neurons larger than the image
 ]
 
 
@@ -88,6 +89,7 @@ DIST_SHAPES = [
     (3, 1, 30, 20, 1024, False, 15, capi.CIRCULAR),       # eight
     (5, 1, 160, 226, 8, True, 113, capi.QUADRATIC),       # neurons too large for an LDS tile: the image in LDS
     (5, 1, 290, 205, 8, True, 40, capi.CIRCULAR),         # ... nothing in LDS
+    (4, 1, 210, 297, 12, True, 148, capi.QUADRATIC),      # ... and neurons larger than the image
     (5, 1, 128, 181, 16, True, 90, capi.QUADRATIC),       # a 128 KiB base rotation in LDS
 ]
 
@@ -371,6 +373,9 @@ FUSED_TRAIN_SHAPES = [
     (4, 1, 160, 226, 8, True, 113, capi.QUADRATIC, capi.UINT8, 2),    # ... but the image fits: interpolated out of LDS
     (3, 1, 160, 226, 8, True, 113, capi.CIRCULAR, capi.UINT16, 2),
     (3, 1, 150, 201, 8, True, 100, capi.QUADRATIC, capi.FLOAT, 2),
+    (3, 1, 210, 260, 8, True, 130, capi.QUADRATIC, capi.UINT8, 2),    # nothing in LDS and neurons larger than the image:
+    (3, 1, 210, 297, 16, True, 148, capi.CIRCULAR, capi.FLOAT, 2),    # tiles of the base rotation that lie beyond the image
+    (2, 2, 204, 230, 4, False, 100, capi.QUADRATIC, capi.UINT16, 2),
     (3, 1, 150, 200, 4, True, 200, capi.QUADRATIC, capi.UINT8, 2),    # 40 000 region elements: uint8 sums beyond 31 bits
     (2, 1, 150, 200, 4, False, 190, capi.QUADRATIC, capi.UINT16, 2),
     (2, 1, 100, 257, 4, False, 257, capi.QUADRATIC, capi.UINT8, 2),   # 66 049: beyond the matrix-core path's row length
