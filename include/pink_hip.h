@@ -95,7 +95,11 @@ typedef struct pink_hip_ctx pink_hip_ctx;
 /* Replaces the constructors Trainer.h:211-260 / Mapper.h:134-179 (device allocation,
  * cos/sin tables, circle tables, upload of the update factors).  Argument errors the
  * reference throws (Trainer.h:66-67, Mapper.h:59-66, CudaLib/generate_rotated_images.h:51,120)
- * are reported here with the same text. */
+ * are reported here with the same text.
+ * Limits of this library (PINK_HIP_EINVAL): in the integer modes a sum of squared differences
+ * must stay below 2^48 and the variants below 65536 (a key is sum << 16 | variant), i.e. uint16
+ * regions of at most 65538 elements, uint8 regions of any practical size; an image or a neuron
+ * holds fewer than 2^31 floats. */
 int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg);
 void pink_hip_destroy(pink_hip_ctx *ctx);
 
