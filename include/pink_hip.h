@@ -101,6 +101,11 @@ typedef struct pink_hip_ctx pink_hip_ctx;
  * regions of at most 65538 elements, uint8 regions of any practical size; an image or a neuron
  * holds fewer than 2^31 floats. */
 int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg);
+/* The argument checks of pink_hip_create alone (the throws of Trainer.h:66-67, Mapper.h:59-66 and
+ * CudaLib/generate_rotated_images.h:51,120), without touching a device: for callers that, like the
+ * reference's constructors, report argument errors before the first image is seen.  Message through
+ * pink_hip_last_error(NULL). */
+int pink_hip_check_config(const pink_hip_config *cfg);
 void pink_hip_destroy(pink_hip_ctx *ctx);
 
 /* Message of the last failing call on `ctx` (or of the last failing

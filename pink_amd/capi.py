@@ -29,7 +29,7 @@ EXPORTS = (
     "pink_hip_distance", "pink_hip_region_size", "pink_hip_distance_kernel", "pink_hip_set_profiling",
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
     "pink_hip_make_update_factors", "pink_hip_layout_distances", "pink_hip_shuffled_order",
-    "pink_hip_fill_random_uniform", "pink_hip_update_counts",
+    "pink_hip_fill_random_uniform", "pink_hip_update_counts", "pink_hip_check_config",
 )
 
 
@@ -62,6 +62,7 @@ def lib():
         vp, u32, f32p, u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
         L.pink_hip_abi_version.restype = C.c_int
         L.pink_hip_create.argtypes = [C.POINTER(vp), C.POINTER(Config)]
+        L.pink_hip_check_config.argtypes = [C.POINTER(Config)]
         L.pink_hip_destroy.argtypes = [vp]
         L.pink_hip_destroy.restype = None
         L.pink_hip_last_error.argtypes = [vp]
@@ -157,6 +158,17 @@ def fill_random_uniform(length, seed):
     if rc != 0:
         raise PinkError(rc, "pink_hip_fill_random_uniform: invalid argument")
     return out
+
+
+def check_config(som_size, channels, image_dim, neuron_dim, num_rot, use_flip, ed_dim, ed_shape=QUADRATIC,
+                 ed_type=FLOAT, interpolation=BILINEAR):
+    """The argument checks of a context's creation without touching a device; raises PinkError as
+    the creation would."""
+    cfg = Config(som_size, channels, image_dim, neuron_dim, num_rot, int(bool(use_flip)), interpolation,
+                 ed_dim, ed_shape, ed_type, None, 0, 0, KERNEL_AUTO)
+    rc = lib().pink_hip_check_config(C.byref(cfg))
+    if rc != 0:
+        raise PinkError(rc, lib().pink_hip_last_error(None).decode())
 
 
 class Context:

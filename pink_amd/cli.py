@@ -33,6 +33,13 @@ SHORT_OPTIONS = {"v": ("version", False), "d": ("neuron-dimension", True), "l": 
                  "h": ("help", False), "f": ("dist-func", True)}
 
 
+def _atoi(text):
+    """std::atoi: optional sign and leading digits, 0 when there are none."""
+    import re
+    m = re.match(r"\s*([+-]?\d+)", text)
+    return int(m.group(1)) if m else 0
+
+
 def _uint32(text):
     try:
         value = int(text)
@@ -143,7 +150,7 @@ class InputData:
         elif name == "seed":
             self.seed = _uint32(value)
         elif name == "progress":
-            self.max_number_of_progress_prints = int(value)
+            self.max_number_of_progress_prints = _atoi(value)      # std::atoi (InputData.cpp:181)
         elif name == "numrot":
             self.number_of_rotations = _uint32(value)
             if self.number_of_rotations == 0 or (self.number_of_rotations != 1 and self.number_of_rotations % 4):

@@ -681,9 +681,8 @@ __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict
             if (c < nchunks) {
                 const v4f *cur = s_rot[c & 1] + lane * (kDistRow / 4);
                 float bv[HB];
-                // (a VALU write of a DPP source needs two idle slots before the DPP read; the no-op
-                // makes that independent of what the compiler schedules next to this point)
-                asm volatile("s_nop 1");
+                // (a VALU write of a DPP source needs two idle slots before the DPP read: every
+                // generated block begins with the no-op that provides them)
                 PINK_SLAB(0) PINK_SLAB(1) PINK_SLAB(2) PINK_SLAB(3)
                 if (c + 1 < nchunks) {
                     v4f *nx = s_rot[(c + 1) & 1];
@@ -2056,10 +2055,9 @@ int pink_hip_abi_version(void) { return PINK_HIP_ABI_VERSION; }
 
 const char *pink_hip_last_error(const pink_hip_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
 
-int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
+int pink_hip_check_config(const pink_hip_config *cfg)
 {
-    if (!out || !cfg) return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: null argument");
-    *out = nullptr;
+    if (!cfg) return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_check_config: null argument");
     // SelfOrganizingMapLib/Trainer.h:66-67, Mapper.h:59-62
     if (cfg->num_rot == 0 || (cfg->num_rot != 1 && cfg->num_rot % 4 != 0))
         return fail(nullptr, PINK_HIP_EINVAL, "Number of rotations must be 1 or larger then 1 and divisible by 4");
@@ -2076,6 +2074,14 @@ int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
     if ((uint64_t)cfg->image_dim * cfg->image_dim >= (1ull << 31) ||
         (uint64_t)cfg->channels * cfg->neuron_dim * cfg->neuron_dim >= (1ull << 31))
         return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: image or neuron too large");
+    return PINK_HIP_OK;
+}
+
+int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg)
+{
+    if (!out || !cfg) return fail(nullptr, PINK_HIP_EINVAL, "pink_hip_create: null argument");
+    *out = nullptr;
+    TRY(pink_hip_check_config(cfg));
 
     pink_hip_ctx *ctx = new (std::nothrow) pink_hip_ctx();
     if (!ctx) return fail(nullptr, PINK_HIP_ENOMEM, "pink_hip_create: out of host memory");
@@ -2302,6 +2308,7 @@ int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_i
 {
     if (!ctx || (n_images && (!dev_images || !dev_heatmap_out)))
         return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device: null argument");
+    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map: context was created with update factors (a trainer)");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     for (uint32_t done = 0; done < n_images; done += ctx->Bcap) {
         const uint32_t B = std::min(ctx->Bcap, n_images - done);
@@ -2317,6 +2324,7 @@ int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
 {
     if (!ctx || (n_images && (!host_images || !host_heatmap_out)))
         return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map: null argument");
+    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map: context was created with update factors (a trainer)");
     if (n_images == 0) return PINK_HIP_OK;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     const size_t img_bytes = (size_t)ctx->isz * sizeof(float);

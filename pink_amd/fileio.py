@@ -190,7 +190,8 @@ def read_rot_flip_file(path):
 def initial_som(som_layout, som_dims, neuron_dims, init="zero", seed=1234, som_file=None):
     """The SOM the reference starts training from (SOM.h:69-98), as (number_of_neurons, prod(neuron_dims))
     float32: "zero"; "random" = fill_random_uniform(seed); "random_with_preferred_direction" = the same with
-    the diagonal of the first neuron_dims[-1] x neuron_dims[-1] block of every neuron set to 1; "file" = the
+    the diagonals of the first <number of neurons> planes of neuron_dims[-1] x neuron_dims[-1] set to 1
+    (one per neuron for single-channel neurons); "file" = the
     weights of `som_file`, found as the reference finds them: behind the text header and 9 +
     <SOM dimensionality> integers (SOM.h:94, which assumes two neuron dimensions)."""
     from . import capi
@@ -204,8 +205,13 @@ def initial_som(som_layout, som_dims, neuron_dims, init="zero", seed=1234, som_f
     if init in ("random", "random_with_preferred_direction"):
         som = capi.fill_random_uniform(n * per_neuron, seed).reshape(n, per_neuron)
         if init == "random_with_preferred_direction":
+            # SOM.h:83-86 indexes the flat weights as n * d*d + i * d + i for n < number of neurons, without
+            # the channel count: for C channels that is the diagonal of the first n planes of d x d, not one
+            # plane per neuron
             d = int(neuron_dims[-1])
-            som[:, np.arange(d) * d + np.arange(d)] = 1.0
+            flat = som.reshape(-1)
+            i = np.arange(d)
+            flat[(np.arange(n)[:, None] * (d * d) + i * d + i).ravel()] = 1.0
         return som
     if init == "file":
         with open(som_file, "rb") as f:

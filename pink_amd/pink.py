@@ -199,13 +199,11 @@ class _Device:
         self.image_dim = None
         self.update_factors = update_factors
         self.counts_base = None
-        # argument errors surface at construction, as in the reference: probe with the neuron size
-        # (the library checks its arguments before it touches a device)
-        try:
-            self._context(self.neuron_dim).close()
-        except capi.PinkError as e:
-            if e.status == -1:
-                raise
+        # argument errors surface at construction, as in the reference; the image size is not known
+        # yet and takes no part in these checks, so the neuron size stands in for it
+        a = self.args
+        capi.check_config(som.number_of_neurons, self.channels, self.neuron_dim, self.neuron_dim, a["num_rot"],
+                          a["use_flip"], a["ed_dim"], a["ed_shape"], a["ed_type"], a["interpolation"])
 
     def _context(self, image_dim):
         return capi.Context(self.som.number_of_neurons, self.channels, image_dim, self.neuron_dim, **self.args)

@@ -51,6 +51,10 @@ def test_options(tmp_path):
     assert c.init == "file" and c.write_rot_flip and c.rot_flip_filename == "rot.bin"      # --map forces FILEINIT
     f = c.distribution()
     assert (f.kind, f.sigma, f.damping) == (capi.MEXICAN_HAT, 2.0, 0.05)
+    # --progress goes through std::atoi (InputData.cpp:181): leading digits count, anything else is 0
+    for text, want in (("12abc", 12), ("abc", 0), (" 7", 7), ("2.9", 2)):
+        c = cli.InputData().parse(["--train", str(tmp_path / "data.bin"), "x.bin", "--progress", text])
+        assert c.max_number_of_progress_prints == want
 
 
 @pytest.mark.parametrize("argv,text", [

@@ -152,6 +152,14 @@ def test_initial_som_kinds(tmp_path):
     plain = O.fill_random_uniform(4 * 9, 5).reshape(4, 9)
     assert np.array_equal(d[:, [0, 4, 8]], np.ones((4, 3), np.float32))
     assert np.array_equal(np.delete(d, [0, 4, 8], axis=1), np.delete(plain, [0, 4, 8], axis=1))
+    # three channels: the reference's flat index n * d*d + i*d + i (SOM.h:83-86) has no channel factor, so the
+    # diagonals of the first <number of neurons> planes are set, wherever they fall
+    d3 = fileio.initial_som("cartesian-2d", (2, 2), (3, 2, 2), "random_with_preferred_direction", seed=5)
+    want = O.fill_random_uniform(4 * 12, 5)
+    for n_ in range(4):
+        for i_ in range(2):
+            want[n_ * 4 + i_ * 2 + i_] = 1.0
+    assert np.array_equal(d3.ravel(), want)
     # "file": weights behind the header and 9 + <SOM dimensionality> integers
     w = np.arange(4 * 9, dtype=np.float32).reshape(4, 9)
     fileio.write_som_file(tmp_path / "init.bin", w, "cartesian-2d", (2, 2), (3, 3), b"# x\n# END OF HEADER\n")
