@@ -1,18 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the PINK hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0]
 
-A step is one pass of the hot path over one batch of synthetic input: the whole
-image set of the workload, mapped (cfg1) or trained in order (cfg0/2/3/4), with the
-images already resident in HBM when the timed region starts.  Default workload: cfg1
-(mapping 20 000 images, uint8 distances, 720 variants) with the SOM obtained by
-training cfg0 for one epoch on the GPU first (untimed).
+A step is one pass of the hot path over one batch of synthetic input: the image set of the
+workload trained in order (cfg0/2/3/4: every image sees the weights the image before it left,
+the final SOM copied back to the host at the end of the step, Trainer::update_som) or mapped
+(cfg1), with the images already resident in HBM when the timed region starts.
 
-Prints ONE JSON line with the throughput, a `roofline` object for the kernel class
-that takes most of the time (durations from HIP events recorded on the library's own
-stream around every launch) and a `cpu_baseline` object (the CPU oracle timed on a
-bounded sample of the same workload on this host's cores).
+Default workload: cfg0, the configuration the metric is quoted on -- training a 10x10 SOM in
+float32 on 2 000 images of 64x64 with 360 rotations x flip (720 variants).  The same JSON line
+carries, under `all_configs`, the other four configurations on a bounded number of images each
+(fixed step counts, whatever --steps says).
+
+Prints ONE JSON line with the throughput, a `roofline` object for the kernel class that takes
+most of the time (durations from HIP events recorded on the library's own stream around every
+launch, in a pass of the same step right after the timed one), a `cpu_baseline` object (the CPU
+oracle timed on a bounded sample of the same workload on this host's cores) and
+`host_inclusive` (the same step through the host-pointer entry points: H2D of the images and D2H
+of the results inside the clock; never `value`).
 """
 import argparse
 import json
@@ -27,29 +33,35 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
-FP32_PEAK_TFLOPS = 157.3       # MI355X vector fp32 (packed FMA), published
+FP32_PEAK_TFLOPS = 157.3       # MI355X fp32 (vector with packed FMA, and fp32 MFMA), published
 
 DTYPE_NAME = {0: "f32", 1: "u16", 2: "u8"}
 
-
-# Peaks measured on the MI355X box used for this work with small microbenchmarks (independent
-# MFMA / fma streams on all CUs): the clock settles near 2.0-2.2 GHz under load.  Reported next to
-# the published figures, never instead of them.
+# Peaks measured on an MI355X of this pool with small microbenchmarks (independent MFMA / fma
+# streams on all CUs): the clock settles near 2.0-2.2 GHz under load.  Reported next to the
+# published figures, never instead of them.
 MEASURED_INT8_MFMA_TOPS = 4130.0
 MEASURED_FMA_NOPACK_TFLOPS = 72.5
 
-# HBM bytes per image from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/cfg1_map_u8_hbm_traffic.txt),
-# scaled by the same counters' readings for a 256 MiB device-to-device copy (FETCH x2.0, WRITE x1.0).
-MEASURED_TRAFFIC_PER_IMAGE = {
-    ("cfg1", 3, "rotate"): 49.2e3 + 103.8e3,     # image + part of the geometry table read; units written
-    ("cfg1", 3, "distance"): 107.3e3 + 0.8e3,    # units read once; keys written
+# HBM bytes per image of one kernel class from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
+# by what the same counter reads for a device-to-device copy of known size; (bytes, the summary
+# under profiles/ that holds the readings).  Not measured in the run that prints the line.
+COUNTER_TRAFFIC_PER_IMAGE = {
+    ("cfg1", "rotate"): (49.2e3 + 103.8e3, "profiles/cfg1_map_u8_hbm_traffic.txt"),
+    ("cfg1", "distance"): (107.3e3 + 0.8e3, "profiles/cfg1_map_u8_hbm_traffic.txt"),
 }
+
+# Images per step of the workloads that ride along in `all_configs` (the headline workload always
+# runs its whole image set): bounded so that the default run stays within minutes; training is
+# sequential, so the rate per image does not depend on how many follow.
+SIDE_IMAGES = {"cfg0": 2000, "cfg1": 20000, "cfg2": 1500, "cfg3": 600, "cfg4": 20000}
+SIDE_STEPS = {"cfg0": (1, 3), "cfg1": (5, 20), "cfg2": (1, 2), "cfg3": (1, 2), "cfg4": (1, 2)}   # (warm-up, timed)
 
 
 def algorithmic_per_image(w, E, path):
     """Algorithmic bytes / operations per image for each kernel class.  `path` is the distance
-    kernel in use (capi.KERNEL_VALU / _MFMA / _MFMA_SYM): the matrix-core paths never write the
-    float variants, their rotation kernel emits the packed distance operand directly."""
+    kernel in use (capi.KERNEL_VALU / _MFMA / _MFMA_SYM / _MFMA_GEMM): the matrix-core mapping paths
+    never write the float variants, their rotation kernel emits the packed distance operand directly."""
     elem = {0: 4, 1: 2, 2: 1}[w.ed_type]
     S, R, N = w.neuron_size, w.R, w.som_size
     nrr = max(w.num_rot // 4, 1)
@@ -82,45 +94,63 @@ def algorithmic_per_image(w, E, path):
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps (default: 30 for the mapping workload, whose step takes a few ms, 3 for training)")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 10 mapping, 1 training)")
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
-    ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--host-buffers", action="store_true",
-                    help="also time one step through the host-pointer entry points (PCIe transfers included); "
-                         "reported as `pcie_inclusive`, never as `value`")
-    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma", "mfma_sym", "mfma_gemm"])
-    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
-                    help="also run one plain device-to-device copy of this many MiB (a kernel of known "
-                         "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every figure is a "
-              "single-MI355X figure)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
+def cpu_baseline(w, som0, imgs_host, budget_s, quick=False):
+    """The CPU oracle on a bounded sample of the workload: all host threads, one thread, and, for the
+    integer workloads, the float32 arithmetic that the reference's own CPU path would run on them
+    (it has no integer mode)."""
+    import oracle as O
+    from pink_amd import capi, synthetic
+    F = synthetic.update_factors(w) if w.mode == "train" else None
+    threads = O.num_threads()
 
+    def shape(ed_type):
+        return O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
+                       w.ed_shape, ed_type)
+
+    def run(s, n):
+        t = time.perf_counter()
+        if w.mode == "map":
+            O.map_images(s, som0, imgs_host[:n])
+        else:
+            O.train(s, som0.copy(), imgs_host[:n], F)
+        return time.perf_counter() - t
+
+    def rate(s, nthreads, budget):
+        O.set_num_threads(nthreads)
+        n_all = len(imgs_host)
+        run(s, min(2, n_all))                          # warm-up
+        probe_n = min(4 if nthreads > 1 else 1, n_all)
+        probe = run(s, probe_n)
+        n = int(max(probe_n, min(n_all, budget / max(probe / probe_n, 1e-6))))
+        dt = run(s, n)
+        O.set_num_threads(threads)
+        return n / dt, n, dt
+
+    v, n, dt = rate(shape(w.ed_type), threads, budget_s)
+    out = {"value": round(v, 3), "unit": "images/s", "cores": threads, "kind": "port",
+           "sample": "%d images of %s, %.1f s, OpenMP over rotations" % (n, w.name, dt),
+           "note": "the port keeps the reference's arithmetic and loop order but its parallel loop is leaner than the "
+                   "reference's (one critical section per thread, no std::function call per pair: "
+                   "generate_euclidean_distance_matrix.h:45-56), so it is somewhat faster than the reference's CPU path"}
+    if not quick:
+        v1, n1, dt1 = rate(shape(w.ed_type), 1, budget_s / 3)
+        out["one_thread"] = {"value": round(v1, 3), "sample": "%d images, %.1f s" % (n1, dt1)}
+    if w.ed_type != capi.FLOAT:
+        vf, nf, dtf = rate(shape(capi.FLOAT), threads, budget_s / 3)
+        out["float32_cpu_path"] = {"value": round(vf, 3), "cores": threads, "sample": "%d images, %.1f s" % (nf, dtf),
+                                   "what": "the same workload in float32: the arithmetic the reference's CPU path "
+                                           "uses whatever the distance type (it has no integer mode)"}
+    return out
+
+
+def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclusive, quick_cpu, calibrate_copy=0):
     import torch
     from pink_amd import capi, synthetic
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(3)
     dev = torch.device("cuda:0")
-    w = synthetic.WORKLOADS[args.workload]
-    # a mapping step is a few milliseconds of GPU time: enough of them that the clocks have settled
-    if args.steps is None:
-        args.steps = 30 if w.mode == "map" else 3
-    if args.warmup is None:
-        args.warmup = 10 if w.mode == "map" else 1
-    n_images = args.images or w.n_images
+    w = synthetic.WORKLOADS[name]
     kernel_choice = {"auto": capi.KERNEL_AUTO, "valu": capi.KERNEL_VALU, "mfma": capi.KERNEL_MFMA,
-                     "mfma_sym": capi.KERNEL_MFMA_SYM, "mfma_gemm": capi.KERNEL_MFMA_GEMM}[args.kernel]
-
+                     "mfma_sym": capi.KERNEL_MFMA_SYM, "mfma_gemm": capi.KERNEL_MFMA_GEMM}[kernel]
     t0 = time.time()
     imgs_host = synthetic.images(w, n_images)
     som0 = synthetic.initial_som(w)
@@ -137,12 +167,13 @@ def main():
     E = ctx.region_size
     ctx.set_som(som0)
     d_imgs = torch.from_numpy(imgs_host).to(dev)
-    d_heat = torch.empty((n_images, w.som_size), dtype=torch.float32, device=dev)
-    d_best = torch.empty((n_images, w.som_size), dtype=torch.int32, device=dev)
+    d_heat = torch.empty((n_images, w.som_size), dtype=torch.float32, device=dev) if w.mode == "map" else None
+    d_best = torch.empty((n_images, w.som_size), dtype=torch.int32, device=dev) if w.mode == "map" else None
     d_bmu = torch.empty((n_images,), dtype=torch.int32, device=dev)
+    som_host = np.empty_like(som0)
     torch.cuda.synchronize()
-    if args.calibrate_copy:
-        src = torch.empty(args.calibrate_copy << 20, dtype=torch.uint8, device=dev)
+    if calibrate_copy:
+        src = torch.empty(calibrate_copy << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)            # reads and writes exactly calibrate_copy MiB each
         torch.cuda.synchronize()
@@ -153,42 +184,39 @@ def main():
             ctx.map_device(d_imgs.data_ptr(), n_images, d_heat.data_ptr(), d_best.data_ptr())
         else:
             ctx.train_device(d_imgs.data_ptr(), n_images, d_bmu.data_ptr())
+            ctx.get_som(out=som_host)              # Trainer::update_som(): the weights back on the host
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         if w.mode == "train":
             ctx.set_som(som0)
         step()
     ctx.synchronize()
 
-    # ---- timed region: exactly `steps` steps, nothing but the path's own launches on the stream ----
-    if w.mode == "train":
-        ctx.set_som(som0)
+    # ---- timed region: exactly `steps` steps, nothing but the path's own launches on the stream.
+    # A training step starts from the weights the step before left (a further epoch): resetting them
+    # would put an upload into the clock that the path does not have.
     ctx.set_profiling(False)
     torch.cuda.synchronize()
     ctx.synchronize()
     t_start = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     ctx.synchronize()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_start
     # ---- per-kernel durations: HIP events around every launch, on the context's stream, in a pass of
-    # their own right after the timed one (the event records cost a mapper several per cent of its
-    # throughput and a trainer, with thousands of launches per second, much more)
+    # the same step right after the timed ones (the event records cost a mapper several per cent of its
+    # throughput and a trainer, with tens of thousands of launches per second, much more)
     ctx.set_profiling(True)
-    if w.mode == "map":
-        for _ in range(args.steps):
-            step()
-        prof_images = n_images * args.steps
-        measured = "the %d timed steps repeated with per-launch HIP events" % args.steps
-    else:
-        prof_images = min(n_images, 256)
-        ctx.train_device(d_imgs.data_ptr(), prof_images, d_bmu.data_ptr())
-        measured = "separate pass of %d images with per-launch HIP events" % prof_images
+    prof_steps = steps if w.mode == "map" else 1
+    for _ in range(prof_steps):
+        step()
+    prof_images = n_images * prof_steps
+    measured = "%d step(s) repeated right after the timed ones with per-launch HIP events" % prof_steps
     times = ctx.kernel_times()
     ctx.set_profiling(False)
 
-    value = n_images * args.steps / elapsed
+    value = n_images * steps / elapsed
     path = ctx.distance_kernel
     alg = algorithmic_per_image(w, E, path)
     total_ms = sum(ms for _, ms in times.values()) or 1e-9
@@ -207,105 +235,146 @@ def main():
         # direct float32 form on the vector ALU: subtract + fma per pair element, counted as 2 ops
         bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
-        notes = ("compute bound on the vector ALU, not on MFMA: bit-faithful sequential fma per (neuron, rotation); "
-                 "packed FP32 is disabled in this build, so the attainable rate is half the published "
-                 "157.3 TFLOP/s (measured %.1f TFLOP/s fma)" % MEASURED_FMA_NOPACK_TFLOPS)
-    elif dominant == "distance" and path == capi.KERNEL_MFMA_SYM:
+        notes = ("compute bound on the vector ALU: bit-faithful sequential fma per (neuron, rotation), one subtract + "
+                 "one fma per pair element (counted as 2 operations), which caps this form at a quarter of the published "
+                 "157.3 TFLOP/s with packed FP32 disabled in this build (measured fma rate %.1f TFLOP/s)"
+                 % MEASURED_FMA_NOPACK_TFLOPS)
+    elif dominant == "distance" and path in (capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA_GEMM, capi.KERNEL_MFMA):
         bound, unit, peak = "mfma", "TOP/s", MFMA_INT8_PEAK_TOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
-        notes = "int8 MFMA; measured MFMA peak on this box %.0f TOP/s" % MEASURED_INT8_MFMA_TOPS
+        notes = "int8 MFMA; measured MFMA peak on this pool %.0f TOP/s" % MEASURED_INT8_MFMA_TOPS
+        if w.ed_type == capi.UINT16:
+            notes += "; uint16 runs four byte-plane products per pair element, counted once"
     else:
         bound, unit, peak = "hbm", "GB/s", HBM_PEAK_GBS
         achieved = alg[dominant]["bytes"] * per_s / 1e9
         if dominant == "rotate" and path != capi.KERNEL_VALU:
             notes = ("vector-ALU bound (exact bilinear arithmetic per operand byte), far from HBM: "
                      "algorithmic bytes = image read + packed operand written")
-    traffic = MEASURED_TRAFFIC_PER_IMAGE.get((args.workload, path, dominant))
+    traffic = COUNTER_TRAFFIC_PER_IMAGE.get((name, dominant))
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
         "frac": round(achieved / peak, 5),
-        "traffic": round(traffic * imgs_per_launch) if traffic else None,
+        "traffic": round(traffic[0] * imgs_per_launch) if traffic else None,
         "algorithmic_bytes_per_launch": round(alg[dominant]["bytes"] * imgs_per_launch),
         "avg_launch_ms": round(avg_ms, 6), "launches": launches, "images_per_launch": imgs_per_launch,
         "measured": measured,
         "share_of_kernel_time": round(ms / total_ms, 4),
         "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
+        "kernel_us_per_image": {k: round(v[1] * 1e3 / prof_images, 4) for k, v in times.items()},
         "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries",
                           4: "int8 MFMA GEMM, split k"}[path],
     }
+    if traffic:
+        roofline["traffic_source"] = traffic[1] + " (rocprofv3 counters of an earlier run of this command, not of this run)"
     if notes:
         roofline["note"] = notes
-    # the distance kernel's own fractions, whichever kernel dominates
+    # the HBM-bound kernels by their algorithmic bytes
+    for cls, key in (("rotate", "rotate_kernel"), ("update", "update_kernel")):
+        c_launches, c_ms = times[cls]
+        if c_launches:
+            c_per_s = prof_images / (c_ms * 1e-3)
+            roofline[key] = {"share_of_kernel_time": round(c_ms / total_ms, 4),
+                             "hbm_frac_algorithmic_bytes": round(alg[cls]["bytes"] * c_per_s / 1e9 / HBM_PEAK_GBS, 5),
+                             "us_per_image": round(c_ms * 1e3 / prof_images, 4)}
     d_launches, d_ms = times["distance"]
-    if d_launches:
+    if d_launches and dominant != "distance":
         d_per_s = prof_images / (d_ms * 1e-3)
-        dist = {"ops_per_s": alg["distance"]["ops"] * d_per_s, "share_of_kernel_time": round(d_ms / total_ms, 4)}
-        if w.ed_type == capi.FLOAT:
-            dist["frac_of_fp32_157.3TF"] = round(dist["ops_per_s"] / 1e12 / FP32_PEAK_TFLOPS, 5)
-            dist["frac_of_measured_nopack_fma"] = round(dist["ops_per_s"] / 1e12 / MEASURED_FMA_NOPACK_TFLOPS, 5)
-        else:
-            dist["frac_of_int8_mfma_5POPs"] = round(dist["ops_per_s"] / 1e12 / MFMA_INT8_PEAK_TOPS, 5)
-            dist["hbm_frac_algorithmic_bytes"] = round(alg["distance"]["bytes"] * d_per_s / 1e9 / HBM_PEAK_GBS, 5)
-        dist["ops_per_s"] = round(dist["ops_per_s"] / 1e12, 3)
-        roofline["distance_kernel"] = dist
-    r_launches, r_ms = times["rotate"]
-    if r_launches:
-        r_per_s = prof_images / (r_ms * 1e-3)
-        roofline["rotate_kernel"] = {"share_of_kernel_time": round(r_ms / total_ms, 4),
-                                     "hbm_frac_algorithmic_bytes": round(alg["rotate"]["bytes"] * r_per_s / 1e9 / HBM_PEAK_GBS, 5),
-                                     "us_per_image": round(r_ms * 1e3 / prof_images, 4)}
+        peak_ops = FP32_PEAK_TFLOPS if w.ed_type == capi.FLOAT else MFMA_INT8_PEAK_TOPS
+        roofline["distance_kernel"] = {"share_of_kernel_time": round(d_ms / total_ms, 4),
+                                       "frac": round(alg["distance"]["ops"] * d_per_s / 1e12 / peak_ops, 5),
+                                       "us_per_image": round(d_ms * 1e3 / prof_images, 4)}
 
-    pcie = None
-    if args.host_buffers:
+    host = None
+    if host_inclusive:
+        # the same step through the host-pointer entry points, as the reference's own loop hands images over
+        # (Pink/main_generic.h:87-89): H2D of the images, D2H of the results, the final SOM for a trainer
         if w.mode == "train":
             ctx.set_som(som0)
+        ctx.synchronize()
         t = time.perf_counter()
         if w.mode == "map":
             ctx.map(imgs_host)
         else:
             ctx.train(imgs_host)
+            ctx.get_som(out=som_host)
         dt = time.perf_counter() - t
-        pcie = {"value": round(n_images / dt, 2), "unit": "images/s",
-                "what": "one step through pink_hip_%s with pageable host buffers: H2D of the images, "
-                        "D2H of the results and the device allocations included" % w.mode}
+        host = {"value": round(n_images / dt, 2), "unit": "images/s",
+                "what": "one step through pink_hip_%s with pageable host buffers: H2D of the images and D2H of the "
+                        "results (a trainer: best matches and the final SOM) inside the clock" % w.mode}
 
-    cpu = None
-    if not args.no_cpu_baseline:
-        import oracle as O
-        s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
-                    w.ed_shape, w.ed_type)
-        F = synthetic.update_factors(w) if w.mode == "train" else None
-
-        def cpu_run(n):
-            t = time.perf_counter()
-            if w.mode == "map":
-                O.map_images(s, som0, imgs_host[:n])
-            else:
-                O.train(s, som0.copy(), imgs_host[:n], F)
-            return time.perf_counter() - t
-
-        cpu_run(min(2, n_images))                      # warm-up
-        probe_n = min(4, n_images)
-        probe = cpu_run(probe_n)
-        n_cpu = int(max(probe_n, min(n_images, 12.0 / max(probe / probe_n, 1e-6))))
-        dt = cpu_run(n_cpu)
-        cpu = {"value": round(n_cpu / dt, 3), "unit": "images/s", "cores": O.num_threads(), "kind": "port",
-               "sample": "%d images of %s, %.1f s, OpenMP over rotations" % (n_cpu, w.name, dt)}
-
-    out = {
-        "metric": ("map" if w.mode == "map" else "train") + " images/sec @%d rot x flip" % w.R,
-        "value": round(value, 2), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": DTYPE_NAME[w.ed_type], "data": "synthetic",
-        "config": {"workload": w.name, "mode": w.mode, "images_per_step": n_images, "som_size": w.som_size,
-                   "neuron": [w.channels, w.neuron_dim, w.neuron_dim], "image": [w.channels, w.image_dim, w.image_dim],
-                   "variants": w.R, "region_elements": E, "distance_kernel": args.kernel,
-                   "som": "cfg0 trained 1 epoch on the GPU" if w.mode == "map" else "mt19937(1234) U[0,1)"},
-        "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(setup_s, 2),
-    }
-    if pcie:
-        out["pcie_inclusive"] = pcie
+    cpu = cpu_baseline(w, som0, imgs_host, cpu_budget_s, quick=quick_cpu) if cpu_budget_s > 0 else None
     ctx.close()
+    del d_imgs, d_heat, d_best, d_bmu
+    torch.cuda.empty_cache()
+    return {
+        "metric": ("map" if w.mode == "map" else "train") + " images/sec @%d rot x flip" % w.R,
+        "value": round(value, 2), "unit": "images/s", "steps": steps, "warmup": warmup,
+        "ms_per_step": round(elapsed / steps * 1e3, 4), "dtype": DTYPE_NAME[w.ed_type],
+        "config": {"workload": w.name, "mode": w.mode, "images_per_step": n_images, "images_in_config": w.n_images,
+                   "som_size": w.som_size, "neuron": [w.channels, w.neuron_dim, w.neuron_dim],
+                   "image": [w.channels, w.image_dim, w.image_dim], "variants": w.R, "region_elements": E,
+                   "distance_kernel": kernel,
+                   "som": "cfg0 trained 1 epoch on the GPU" if w.mode == "map" else "mt19937(1234) U[0,1)"},
+        "roofline": roofline, "cpu_baseline": cpu, "host_inclusive": host, "setup_s": round(setup_s, 2),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps of the headline workload (default: 10 for training, 30 for the mapping workload, "
+                         "whose step takes a few ms)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 2 training, 10 mapping)")
+    ap.add_argument("--workload", default="cfg0", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--images", type=int, default=0, help="override the number of images per step")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-all-configs", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-host-inclusive", action="store_true")
+    ap.add_argument("--kernel", default="auto", choices=["auto", "valu", "mfma", "mfma_sym", "mfma_gemm"])
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run one plain device-to-device copy of this many MiB (a kernel of known "
+                         "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every figure is a "
+              "single-MI355X figure)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from pink_amd import synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    w = synthetic.WORKLOADS[args.workload]
+    # a mapping step is a few milliseconds of GPU time: enough of them that the clocks have settled
+    if args.steps is None:
+        args.steps = 30 if w.mode == "map" else 10
+    if args.warmup is None:
+        args.warmup = 10 if w.mode == "map" else 2
+    cpu_budget = 0.0 if args.no_cpu_baseline else 10.0
+    head = run_workload(args.workload, args.steps, args.warmup, args.images or w.n_images, args.kernel, cpu_budget,
+                        not args.no_host_inclusive, False, args.calibrate_copy)
+    out = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic", "config": head["config"],
+        "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "host_inclusive": head["host_inclusive"],
+        "setup_s": head["setup_s"],
+    }
+    if not args.no_all_configs:
+        side = {}
+        for name in ("cfg0", "cfg1", "cfg2", "cfg3", "cfg4"):
+            if name == args.workload:
+                continue
+            wu, st = SIDE_STEPS[name]
+            r = run_workload(name, st, wu, min(SIDE_IMAGES[name], synthetic.WORKLOADS[name].n_images), "auto",
+                             0.0 if args.no_cpu_baseline else 5.0, not args.no_host_inclusive, True)
+            side[name] = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "config",
+                                            "roofline", "cpu_baseline", "host_inclusive")}
+        out["all_configs"] = side
     print(json.dumps(out))
 
 

@@ -232,6 +232,10 @@ def num_threads():
     return int(lib().pink_oracle_num_threads())
 
 
+def set_num_threads(n):
+    lib().pink_oracle_set_num_threads(C.c_int(int(n)))
+
+
 def fill_random_uniform(n, seed):
     a = np.empty(n, np.float32)
     lib().pink_oracle_fill_random_uniform(_p(a, C.c_float), C.c_size_t(n), C.c_uint32(seed))

@@ -648,6 +648,16 @@ void pink_oracle_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order)
     for (uint32_t i = 1; i < n; ++i) swap_u32(&order[i], &order[uniform_below(&g, (uint64_t)i + 1)]);
 }
 
+/* Number of threads for the OpenMP loops above (the reference's --numthreads, UtilitiesLib/InputData.cpp:485). */
+void pink_oracle_set_num_threads(int n)
+{
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
 /* Threads the OpenMP loops above will use (1 without OpenMP). */
 int pink_oracle_num_threads(void)
 {

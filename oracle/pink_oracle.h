@@ -129,6 +129,7 @@ void pink_oracle_mt19937_raw(uint32_t seed, uint32_t *out, size_t n);
 void pink_oracle_shuffled_order(uint64_t seed, uint32_t n, uint32_t *order);
 
 int pink_oracle_num_threads(void);
+void pink_oracle_set_num_threads(int n);
 
 #ifdef __cplusplus
 }

@@ -231,8 +231,10 @@ class Context:
         assert som.size == self.N * self.S
         self._check(self._L.pink_hip_set_som(self._h, _f32(som)))
 
-    def get_som(self):
-        out = np.empty((self.N, self.S), np.float32)
+    def get_som(self, out=None):
+        if out is None:
+            out = np.empty((self.N, self.S), np.float32)
+        assert out.dtype == np.float32 and out.flags.c_contiguous and out.size == self.N * self.S
         self._check(self._L.pink_hip_get_som(self._h, _f32(out)))
         return out
 

@@ -152,8 +152,10 @@ def update_factors(w):
     return capi.make_update_factors(w.layout, w.som_dims, w.functor, w.sigma, w.damping, -1.0)
 
 
-def make_context(w, trainer=None, **kw):
-    """A device context shaped for workload w (a trainer for "train" workloads)."""
+def make_context(w, trainer=None, ed_type=None, **kw):
+    """A device context shaped for workload w (a trainer for "train" workloads), optionally with
+    another distance type."""
     trainer = (w.mode == "train") if trainer is None else trainer
     return capi.Context(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim,
-                        w.ed_shape, w.ed_type, update_factors(w) if trainer else None, **kw)
+                        w.ed_shape, w.ed_type if ed_type is None else ed_type,
+                        update_factors(w) if trainer else None, **kw)
