@@ -144,6 +144,21 @@ int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
 int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images,
                         float *dev_heatmap_out, uint32_t *dev_best_rot_out);
 
+/* pink_hip_map_device for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments and results as pink_hip_map_device, but the per-group buffers of the call (argmin keys,
+ * packed variant operand, variant norms, float variants where a kernel of its own packs them) are taken
+ * from a static device array of PINK_HIP_STATIC_SCRATCH_BYTES that every GPU holds from the moment the
+ * library is loaded until the process ends, not from the context's own allocations; the call itself
+ * allocates and frees nothing and clears the part of the array it uses with a kernel.  Images are
+ * processed in groups of as many as fit the array; PINK_HIP_EINVAL when a single image of the context
+ * does not fit (the message says how many bytes it needs), PINK_HIP_ESTATE on a trainer or while
+ * per-kernel timing is on (event records allocate).  All contexts on a GPU share the one array: calls
+ * that overlap on the same GPU (two contexts, two streams) race; calls one after the other are fine. */
+#define PINK_HIP_STATIC_SCRATCH_BYTES (32u << 20)
+int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images,
+                               float *dev_heatmap_out, uint32_t *dev_best_rot_out);
+
 /* Wait for everything queued on the context's stream. */
 int pink_hip_synchronize(pink_hip_ctx *ctx);
 

@@ -30,6 +30,7 @@ EXPORTS = (
     "pink_hip_kernel_times", "pink_hip_device_info", "pink_hip_som_size",
     "pink_hip_make_update_factors", "pink_hip_layout_distances", "pink_hip_shuffled_order",
     "pink_hip_fill_random_uniform", "pink_hip_update_counts", "pink_hip_check_config",
+    "pink_hip_map_device_static",
 )
 
 
@@ -74,6 +75,7 @@ def lib():
         L.pink_hip_train_device.argtypes = [vp, vp, u32, vp]
         L.pink_hip_map.argtypes = [vp, f32p, u32, f32p, u32p]
         L.pink_hip_map_device.argtypes = [vp, vp, u32, vp, vp]
+        L.pink_hip_map_device_static.argtypes = [vp, vp, u32, vp, vp]
         L.pink_hip_synchronize.argtypes = [vp]
         L.pink_hip_rotate.argtypes = [vp, f32p, f32p]
         L.pink_hip_distance.argtypes = [vp, f32p, f32p, C.POINTER(C.c_int64), u32p]
@@ -271,6 +273,10 @@ class Context:
 
     def map_device(self, dev_images_ptr, n, dev_heat_ptr, dev_best_ptr=None):
         self._check(self._L.pink_hip_map_device(self._h, dev_images_ptr, n, dev_heat_ptr, dev_best_ptr))
+
+    def map_device_static(self, dev_images_ptr, n, dev_heat_ptr, dev_best_ptr=None):
+        """map_device out of the library's static scratch array: allocates nothing."""
+        self._check(self._L.pink_hip_map_device_static(self._h, dev_images_ptr, n, dev_heat_ptr, dev_best_ptr))
 
     def synchronize(self):
         self._check(self._L.pink_hip_synchronize(self._h))

@@ -28,8 +28,18 @@
 #include <type_traits>
 #include <vector>
 
+#include <mutex>
+
 #include "mfma_u8_sym.h"
 #include "pink_hip.h"
+
+// Scratch of pink_hip_map_device_static, the entry point for callers that cannot allocate: the
+// per-group buffers of a mapping call (argmin keys, the packed variant operand, variant norms, float
+// variants where a kernel of its own packs them) live in this array instead of in buffers the
+// context allocated.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends; host code reaches it only through the address hipGetSymbolAddress returns for the
+// current device (the name below is a host-side stand-in, not a device address).
+static __device__ __align__(256) unsigned char scratch[PINK_HIP_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -57,6 +67,13 @@ __device__ __forceinline__ unsigned long long wave_min_u64(unsigned long long v)
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+
+// Zero `n16` 16-byte words (a kernel, not a memset: a caller may be capturing the stream into a graph).
+__global__ __launch_bounds__(256) void k_fill_zero(v4i *__restrict__ p, size_t n16)
+{
+    const v4i z = {0, 0, 0, 0};
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n16; t += (size_t)gridDim.x * blockDim.x) p[t] = z;
+}
 
 // q = T(x * factor) truncated, saturated to [0, factor] (CudaLib/copy_and_transform_kernel.h:27-28)
 __device__ __forceinline__ int32_t quantise(float x, float factor)
@@ -1186,6 +1203,8 @@ struct pink_hip_ctx {
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
 
+    unsigned char *static_scratch = nullptr;   // this device's copy of the file-scope scratch array
+
     bool profiling = false;
     std::vector<EventPair> events;
     std::vector<hipEvent_t> event_pool;
@@ -1577,10 +1596,29 @@ int free_all(pink_hip_ctx *ctx)
     return PINK_HIP_OK;
 }
 
+// The address of the file-scope scratch array on the current device, asked for once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[kMaxDevices] = {};
+
+int resolve_static_scratch(pink_hip_ctx *ctx)
+{
+    if (ctx->device < 0 || ctx->device >= kMaxDevices) return fail(ctx, PINK_HIP_EINVAL, "device ordinal out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[ctx->device]) {
+        void *p = nullptr;
+        HIP_TRY(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[ctx->device] = (unsigned char *)p;
+    }
+    ctx->static_scratch = g_scratch_ptr[ctx->device];
+    return PINK_HIP_OK;
+}
+
 int init_ctx(pink_hip_ctx *ctx)
 {
     const pink_hip_config &c = ctx->cfg;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
+    TRY(resolve_static_scratch(ctx));
     HIP_TRY(ctx, hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
 
     // Rotation tables: cos/sin of i * 2pi/num_rot in float, as the CPU evaluates them
@@ -2317,6 +2355,94 @@ int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_i
                          dev_best_rot_out ? dev_best_rot_out + (size_t)done * ctx->N : nullptr, true));
     }
     return PINK_HIP_OK;
+}
+
+// The per-group buffers of a mapping call, per image, in the order they are carved out of the static
+// scratch (every piece starts on a 256-byte boundary).
+struct StaticPieces {
+    size_t key = 0, Pb = 0, nb = 0, gPb = 0, gnb = 0, rot = 0, rotT = 0;
+    size_t per_image() const { return key + Pb + nb + gPb + gnb + rot + rotT; }
+};
+
+StaticPieces static_pieces(const pink_hip_ctx *ctx)
+{
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    StaticPieces p;
+    p.key = up((size_t)ctx->N * sizeof(unsigned long long));
+    if (ctx->mfma_sym) {
+        p.Pb = up((size_t)ctx->RTP * pink_sym::unit_bytes(ctx->KSs));
+    } else if (ctx->mfma) {
+        p.Pb = up((size_t)ctx->RT * ctx->KS * 1024);
+        p.nb = up((size_t)ctx->RT * 32 * sizeof(int));
+    } else if (ctx->gemm) {
+        const size_t planes = ctx->cfg.ed_type == PINK_HIP_UINT16 ? 2 : 1;
+        p.gPb = up(planes * (ctx->Rp / 32) * ctx->gKS * 1024);
+        p.gnb = up((size_t)ctx->Rp * sizeof(long long));
+    } else {
+        p.rotT = up((size_t)ctx->Epad * ctx->Rpad * 4);
+    }
+    if (!ctx->mfma && !ctx->mfma_sym && !ctx->fused_pack) p.rot = up((size_t)ctx->R * ctx->S * sizeof(float));
+    return p;
+}
+
+int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, float *dev_heatmap_out,
+                               uint32_t *dev_best_rot_out)
+{
+    if (!ctx || (n_images && (!dev_images || !dev_heatmap_out)))
+        return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device_static: null argument");
+    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map: context was created with update factors (a trainer)");
+    if (ctx->profiling)
+        return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: per-kernel timing creates events; switch it off");
+    if (!ctx->static_scratch) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: no static scratch on this device");
+    const StaticPieces pc = static_pieces(ctx);
+    const size_t per_image = pc.per_image();
+    if (per_image > PINK_HIP_STATIC_SCRATCH_BYTES)
+        return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device_static: one image of this context needs " + std::to_string(per_image) +
+                                          " bytes of scratch, the static scratch holds " +
+                                          std::to_string((size_t)PINK_HIP_STATIC_SCRATCH_BYTES));
+    if (n_images == 0) return PINK_HIP_OK;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    const uint32_t B = (uint32_t)std::min<size_t>({(size_t)ctx->Bcap, PINK_HIP_STATIC_SCRATCH_BYTES / per_image, (size_t)n_images});
+
+    // the scratch keeps what the last call (of any context on this GPU) left: rows beyond the last variant
+    // and elements beyond the region must read as zero, so the part this call uses starts from zero
+    const size_t used = (size_t)B * per_image;
+    hipLaunchKernelGGL(k_fill_zero, dim3((uint32_t)std::min<size_t>((used / 16 + 255) / 256, 2048)), dim3(256), 0, ctx->stream,
+                       (v4i *)ctx->static_scratch, used / 16);
+    TRY(launch_check(ctx, "k_fill_zero"));
+
+    // the kernels take the scratch where they take the context's own buffers in pink_hip_map_device
+    struct Saved {
+        unsigned long long *key; signed char *Pb; int *nb; v4i *gPb; long long *gnb; float *rot; void *rotT;
+        uint32_t Bcap, gslices, gks_per;
+    } const saved{ctx->d_key, ctx->d_Pb, ctx->d_nb, ctx->d_gPb, ctx->d_gnb, ctx->d_rot, ctx->d_rotT, ctx->Bcap, ctx->gslices, ctx->gks_per};
+    unsigned char *at = ctx->static_scratch;
+    auto carve = [&](size_t bytes_per_image) { unsigned char *p = at; at += (size_t)B * bytes_per_image; return p; };
+    ctx->d_key = (unsigned long long *)carve(pc.key);
+    if (pc.Pb) ctx->d_Pb = (signed char *)carve(pc.Pb);
+    if (pc.nb) ctx->d_nb = (int *)carve(pc.nb);
+    if (pc.gPb) ctx->d_gPb = (v4i *)carve(pc.gPb);
+    if (pc.gnb) ctx->d_gnb = (long long *)carve(pc.gnb);
+    if (pc.rot) ctx->d_rot = (float *)carve(pc.rot);
+    if (pc.rotT) ctx->d_rotT = carve(pc.rotT);
+    ctx->Bcap = B;
+    if (ctx->gemm) {
+        // a block takes the whole k range of its tile also when a group holds a single image: no partial
+        // sums in memory (the context's own buffer for them is not used here)
+        ctx->gslices = 1;
+        ctx->gks_per = (ctx->gKS + 3) / 4;
+    }
+    int rc = PINK_HIP_OK;
+    for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += B) {
+        const uint32_t b = std::min(B, n_images - done);
+        rc = distance_group(ctx, dev_images + (size_t)done * ctx->isz, b);
+        if (rc == PINK_HIP_OK)
+            rc = run_finalize(ctx, b, dev_heatmap_out + (size_t)done * ctx->N, nullptr,
+                              dev_best_rot_out ? dev_best_rot_out + (size_t)done * ctx->N : nullptr, true);
+    }
+    ctx->d_key = saved.key; ctx->d_Pb = saved.Pb; ctx->d_nb = saved.nb; ctx->d_gPb = saved.gPb; ctx->d_gnb = saved.gnb;
+    ctx->d_rot = saved.rot; ctx->d_rotT = saved.rotT; ctx->Bcap = saved.Bcap; ctx->gslices = saved.gslices; ctx->gks_per = saved.gks_per;
+    return rc;
 }
 
 int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, float *host_heatmap_out,
