@@ -64,7 +64,10 @@ typedef enum {
     PINK_HIP_KERNEL_VALU = 1,      /* integer modes on the vector ALU in exact int32/int64                */
     PINK_HIP_KERNEL_MFMA = 2,      /* uint8 mapper, int8 MFMA, symmetries applied to the image variants   */
     PINK_HIP_KERNEL_MFMA_SYM = 3,  /* uint8 mapper, int8 MFMA, symmetries applied to the SOM once         */
-    PINK_HIP_KERNEL_MFMA_GEMM = 4  /* integer modes, trainer or mapper: split-k int8 MFMA GEMM (uint16 as 4 byte-plane products) */
+    PINK_HIP_KERNEL_MFMA_GEMM = 4, /* integer modes, trainer or mapper: split-k int8 MFMA GEMM (uint16 as 4 byte-plane products) */
+    PINK_HIP_KERNEL_MFMA_F32 = 5   /* float32, trainer or mapper, on request only: |a|^2 + |b|^2 - 2 a.b with float32 MFMA dot
+                                      products -- not the CPU's summation order: distances agree to a relative tolerance, best
+                                      rotations where candidates are not that close, trained weights drift */
 } pink_hip_kernel_choice;
 
 /*
@@ -174,7 +177,7 @@ int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_di
 
 /* Number of elements in the distance region (incl. channels) as the context counts it. */
 uint32_t pink_hip_region_size(const pink_hip_ctx *ctx);
-/* The distance kernel the context runs: PINK_HIP_KERNEL_VALU, _MFMA, _MFMA_SYM or _MFMA_GEMM. */
+/* The distance kernel the context runs: PINK_HIP_KERNEL_VALU, _MFMA, _MFMA_SYM, _MFMA_GEMM or _MFMA_F32. */
 uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx);
 
 /* Per-kernel timing with HIP events on the context's stream.  While enabled every

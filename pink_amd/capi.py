@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libpink_hip.so")
 FLOAT, UINT16, UINT8 = 0, 1, 2
 QUADRATIC, CIRCULAR = 0, 1
 NEAREST_NEIGHBOR, BILINEAR = 0, 1
-KERNEL_AUTO, KERNEL_VALU, KERNEL_MFMA, KERNEL_MFMA_SYM, KERNEL_MFMA_GEMM = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_VALU, KERNEL_MFMA, KERNEL_MFMA_SYM, KERNEL_MFMA_GEMM, KERNEL_MFMA_F32 = 0, 1, 2, 3, 4, 5
 CARTESIAN, HEXAGONAL = 0, 1
 STEP, GAUSSIAN, UNITY_GAUSSIAN, MEXICAN_HAT = 0, 1, 2, 3
 NUM_KERNEL_CLASSES = 5

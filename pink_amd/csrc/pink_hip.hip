@@ -934,6 +934,7 @@ __global__ __launch_bounds__(512) void k_dist_mfma_u8(const v4i *__restrict__ Pa
 }
 
 #include "mfma_int_gemm.inc"
+#include "mfma_f32_gemm.inc"
 
 // ---------------------------------------------------------------------------------
 // BMU search fused with the neuron update (Trainer.h:164-179; CudaLib/update_neurons.h).
@@ -1205,6 +1206,13 @@ struct pink_hip_ctx {
 
     unsigned char *static_scratch = nullptr;   // this device's copy of the file-scope scratch array
 
+    // float32 distances recast as a GEMM on the matrix cores (kernel_choice PINK_HIP_KERNEL_MFMA_F32 only)
+    bool f32gemm = false;
+    uint32_t fKS = 0, fslices = 1, fks_per = 0;
+    v4f *d_fPa = nullptr, *d_fPb = nullptr;
+    double *d_fna = nullptr, *d_fnb = nullptr;
+    float *d_fpart = nullptr;
+
     bool profiling = false;
     std::vector<EventPair> events;
     std::vector<hipEvent_t> event_pool;
@@ -1325,6 +1333,14 @@ bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT
 
 // --- launch groups ---------------------------------------------------------------
 
+// Matrix-core float32 path: fragments and norms of the SOM rows (after every change of the packed rows).
+int run_pack_frag_som(pink_hip_ctx *ctx)
+{
+    hipLaunchKernelGGL(k_pack_frag_f32, dim3(ctx->Np / 32, 1), dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, ctx->d_fPa,
+                       ctx->d_fna, ctx->N, ctx->Epad, (size_t)0, (size_t)0, ctx->Np);
+    return launch_check(ctx, "k_pack_frag_f32");
+}
+
 int run_pack_som(pink_hip_ctx *ctx)
 {
     Timed t(ctx, kClsPack);
@@ -1355,7 +1371,8 @@ int run_pack_som(pink_hip_ctx *ctx)
     else
         hipLaunchKernelGGL(k_pack_som<false>, dim3(blocks), dim3(256), 0, ctx->stream, ctx->d_som, ctx->d_region,
                            ctx->d_somP, ctx->N, ctx->S, ctx->E, ctx->Epad, 1.0f);
-    return launch_check(ctx, "k_pack_som");
+    TRY(launch_check(ctx, "k_pack_som"));
+    return ctx->f32gemm ? run_pack_frag_som(ctx) : PINK_HIP_OK;
 }
 
 // store: kStoreNone, kStoreAll or kStorePair (see k_rotate)
@@ -1415,6 +1432,21 @@ int run_rotate(pink_hip_ctx *ctx, const float *dev_images, uint32_t B, uint32_t 
 
 int run_pack_rot(pink_hip_ctx *ctx, uint32_t B)
 {
+    if (ctx->f32gemm) {
+        // the float rows (written by k_rotate or packed below) also go into fragments, with their norms
+        if (!ctx->fused_pack) {
+            Timed t(ctx, kClsPack);
+            PairSource ps{};
+            if (ctx->pair_pack) { ps.off4 = ctx->d_region4; ps.num_rot = ctx->cfg.num_rot; ps.nrr = std::max(ctx->nrr, 1u); ps.E = ctx->E; }
+            hipLaunchKernelGGL(k_pack_rot_rows, dim3((ctx->Epad + 255) / 256, ctx->Rpad, B), dim3(256), 0, ctx->stream,
+                               ctx->d_rot, ctx->d_region, (float *)ctx->d_rotT, ctx->R, ctx->S, ctx->E, ctx->Epad, ctx->Rpad, ps);
+            TRY(launch_check(ctx, "k_pack_rot_rows"));
+        }
+        Timed t(ctx, kClsPack);
+        hipLaunchKernelGGL(k_pack_frag_f32, dim3(ctx->Rp / 32, B), dim3(256), 0, ctx->stream, (const float *)ctx->d_rotT, ctx->d_fPb,
+                           ctx->d_fnb, ctx->R, ctx->Epad, (size_t)ctx->Epad * ctx->Rpad, (size_t)(ctx->Rp / 32) * ctx->fKS * 64, ctx->Rp);
+        return launch_check(ctx, "k_pack_frag_f32");
+    }
     if (ctx->fused_pack) return PINK_HIP_OK;              // k_rotate wrote the operand already
     Timed t(ctx, kClsPack);
     PairSource ps{};
@@ -1521,9 +1553,34 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
                        ctx->Rp, ctx->gslices, rows_per_chunk, ctx->d_gvariant);
 }
 
+// Distances of B images starting at image slot `slot` on the matrix cores, float32.
+int run_dist_f32gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
+{
+    const uint32_t tiles = (ctx->Rp / 64) * (ctx->Np / 64);
+    const uint32_t slices = B > 1 ? 1 : ctx->fslices;
+    const uint32_t ks_per = B > 1 ? (ctx->fKS + 3) / 4 : ctx->fks_per;
+    GemmFinishF32 fin{};
+    fin.na = ctx->d_fna;
+    fin.nb = ctx->d_fnb + (size_t)slot * ctx->Rp;
+    fin.N = ctx->N; fin.R = ctx->R;
+    unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
+    if (slices == 1) fin.key = key;
+    const v4f *pb = ctx->d_fPb + (size_t)slot * (ctx->Rp / 32) * ctx->fKS * 64;
+    hipLaunchKernelGGL(k_dist_gemm_f32, dim3(tiles * slices, B), dim3(256), 65536, ctx->stream, (const v4f *)ctx->d_fPa, pb, ctx->d_fpart,
+                       ctx->Np, ctx->Rp, ctx->fKS, ks_per, slices, fin);
+    TRY(launch_check(ctx, "k_dist_gemm_f32"));
+    if (slices == 1) return PINK_HIP_OK;
+    const uint32_t rows_per_chunk = 32;
+    hipLaunchKernelGGL(k_dist_finish_f32, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk), dim3(256), 0,
+                       ctx->stream, (const float *)ctx->d_fpart, (const double *)ctx->d_fna, fin.nb, key, ctx->N, ctx->Np, ctx->R,
+                       ctx->Rp, slices, rows_per_chunk);
+    return launch_check(ctx, "k_dist_finish_f32");
+}
+
 int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     Timed t(ctx, kClsDist);
+    if (ctx->f32gemm) return run_dist_f32gemm(ctx, slot, B);
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16) launch_dist_gemm<true>(ctx, slot, B);
         else launch_dist_gemm<false>(ctx, slot, B);
@@ -1592,6 +1649,8 @@ int free_all(pink_hip_ctx *ctx)
     for (hipEvent_t e : ctx->copy_ev) if (e) (void)hipEventDestroy(e);
     if (ctx->copy_stream) (void)hipStreamDestroy(ctx->copy_stream);
     if (ctx->d_counts) (void)hipFree(ctx->d_counts);
+    for (void *p : {(void *)ctx->d_fPa, (void *)ctx->d_fPb, (void *)ctx->d_fna, (void *)ctx->d_fnb, (void *)ctx->d_fpart})
+        if (p) (void)hipFree(p);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     return PINK_HIP_OK;
 }
@@ -1824,6 +1883,22 @@ int init_ctx(pink_hip_ctx *ctx)
         }
     }
 
+    // Float32 distances on the matrix cores: only on request.
+    if (c.kernel_choice == PINK_HIP_KERNEL_MFMA_F32) {
+        if (is_int(ctx)) return fail(ctx, PINK_HIP_EINVAL, "the float32 matrix-core distance kernel needs the float distance type");
+        ctx->f32gemm = true;
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_dist_gemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+        ctx->fKS = ctx->Epad / 8;
+        ctx->Np = round_up(ctx->N, 64);
+        ctx->Rp = round_up(ctx->R, 64);
+        const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
+        // k is cut into slices (blocks per tile) to fill the chip about twice, a wave keeping at least four k-steps
+        uint32_t slices = std::max(1u, 2u * (uint32_t)ctx->num_cu / tiles);
+        slices = std::max(1u, std::min(slices, ctx->fKS / 16));
+        ctx->fks_per = (ctx->fKS + 4 * slices - 1) / (4 * slices);
+        ctx->fslices = (ctx->fKS + 4 * ctx->fks_per - 1) / (4 * ctx->fks_per);
+    }
+
     ctx->Dp = ctx->D | 1u;     // odd (measured at D = 96: 20 % faster than a stride of 96; nothing to gain at 44, 70, 106)
     // the base rotation of a block lives in LDS: up to 158 of the CU's 160 KB (neurons up to 199 pixels wide)
     ctx->use_lds = (size_t)ctx->D * ctx->Dp * sizeof(float) <= kRotateLdsMax;
@@ -1945,6 +2020,13 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
         // rows beyond R and elements beyond the region must read as zero whoever fills the rest
         HIP_TRY(ctx, hipMemset(ctx->d_rotT, 0, B * ctx->Epad * ctx->Rpad * sizeof(uint32_t)));
+        if (ctx->f32gemm) {
+            TRY(dev_alloc(ctx, &ctx->d_fPa, (size_t)(ctx->Np / 32) * ctx->fKS * 64));
+            TRY(dev_alloc(ctx, &ctx->d_fPb, B * (ctx->Rp / 32) * ctx->fKS * 64));
+            TRY(dev_alloc(ctx, &ctx->d_fna, (size_t)ctx->Np));
+            TRY(dev_alloc(ctx, &ctx->d_fnb, B * ctx->Rp));
+            TRY(dev_alloc(ctx, &ctx->d_fpart, (size_t)ctx->fslices * ctx->Rp * ctx->Np));
+        }
     }
     if (ctx->fused_pack) {
         const uint32_t D = ctx->D, DD = D * D;
@@ -2210,6 +2292,7 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
             TRY(run_dist(ctx, b, 1));
             TRY(run_update(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
             if (!ctx->d_inv || (ctx->gemm && !ctx->fused_som)) TRY(run_pack_som(ctx));
+            else if (ctx->f32gemm) { Timed t(ctx, kClsPack); TRY(run_pack_frag_som(ctx)); }
         }
     }
     return PINK_HIP_OK;
@@ -2528,7 +2611,7 @@ uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx)
 {
     if (!ctx) return 0;
     return ctx->mfma_sym ? PINK_HIP_KERNEL_MFMA_SYM : ctx->mfma ? PINK_HIP_KERNEL_MFMA
-         : ctx->gemm ? PINK_HIP_KERNEL_MFMA_GEMM : PINK_HIP_KERNEL_VALU;
+         : ctx->gemm ? PINK_HIP_KERNEL_MFMA_GEMM : ctx->f32gemm ? PINK_HIP_KERNEL_MFMA_F32 : PINK_HIP_KERNEL_VALU;
 }
 
 int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)
