@@ -994,26 +994,39 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         x = rot + (size_t)((q & 1) * vp.nrr + i) * S;
         rev_x = f ^ (q >> 1); rev_y = q >> 1;
     }
-    const RcpDivisor by_DD(vp.D * vp.D), by_D(vp.D);
-    auto source = [&](uint32_t j) {
-        if (!vp.D) return j;
-        uint32_t c, p, px, py;
-        by_DD.divmod(j, c, p);
-        by_D.divmod(p, px, py);
-        return j - p + (rev_x ? vp.D - 1 - px : px) * vp.D + (rev_y ? vp.D - 1 - py : py);
-    };
     float *__restrict__ w = som + (size_t)n * S;
     const uint32_t chunk = (S + parts - 1) / parts;
     const uint32_t j0 = part * chunk, j1 = min(S, j0 + chunk);
+    // Where element j of the variant sits in the stored one: j itself unless rows and/or columns are read
+    // reversed.  A thread's elements are 256 apart, so its (row, column) inside the channel plane moves by a fixed
+    // step with carries instead of two divisions per element (the kernel was half bound by its vector ALU work).
+    const bool reversed = vp.D != 0 && (rev_x | rev_y) != 0;
+    const uint32_t D = max(vp.D, 1u);
+    const uint32_t step_x = 256u / D, step_y = 256u % D;
+    uint32_t px = 0, py = 0;                      // of the next element this thread loads
+    if (reversed) {
+        const RcpDivisor by_DD(D * D), by_D(D);
+        uint32_t c, p;
+        by_DD.divmod(j0 + tid, c, p);
+        by_D.divmod(p, px, py);
+    }
     float wv[U], xv[U];
     uint32_t kk[U];
     auto load_round = [&](uint32_t jb) {
 #pragma unroll
         for (uint32_t u = 0; u < U; ++u) {
             const uint32_t j = jb + 256 * u;
+            uint32_t src = j;
+            if (reversed) {
+                src = j - (px * D + py) + (rev_x ? D - 1 - px : px) * D + (rev_y ? D - 1 - py : py);
+                py += step_y;
+                px += step_x + (py >= D ? 1u : 0u);
+                py -= py >= D ? D : 0u;
+                while (px >= D) px -= D;           // (past the end of a channel plane: the next one; twice for D < 16)
+            }
             if (j < j1) {
                 wv[u] = w[j];
-                xv[u] = x[source(j)];
+                xv[u] = x[src];
                 kk[u] = inv ? inv[j] : 0xffffffffu;
             }
         }
