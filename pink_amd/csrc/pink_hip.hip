@@ -1002,10 +1002,12 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     // step with carries instead of two divisions per element (the kernel was half bound by its vector ALU work).
     const bool reversed = vp.D != 0 && (rev_x | rev_y) != 0;
     const uint32_t D = max(vp.D, 1u);
+    const RcpDivisor by_DD(D * D), by_D(D);
+    // (a slice of a single round, small neurons spread over many blocks: the divisions are as cheap as the stepping)
+    const bool stepping = reversed && j1 - j0 > 256 * U;
     const uint32_t step_x = 256u / D, step_y = 256u % D;
     uint32_t px = 0, py = 0;                      // of the next element this thread loads
-    if (reversed) {
-        const RcpDivisor by_DD(D * D), by_D(D);
+    if (stepping) {
         uint32_t c, p;
         by_DD.divmod(j0 + tid, c, p);
         by_D.divmod(p, px, py);
@@ -1017,12 +1019,17 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         for (uint32_t u = 0; u < U; ++u) {
             const uint32_t j = jb + 256 * u;
             uint32_t src = j;
-            if (reversed) {
+            if (stepping) {
                 src = j - (px * D + py) + (rev_x ? D - 1 - px : px) * D + (rev_y ? D - 1 - py : py);
                 py += step_y;
                 px += step_x + (py >= D ? 1u : 0u);
                 py -= py >= D ? D : 0u;
                 while (px >= D) px -= D;           // (past the end of a channel plane: the next one; twice for D < 16)
+            } else if (reversed) {
+                uint32_t c, p, qx, qy;
+                by_DD.divmod(j, c, p);
+                by_D.divmod(p, qx, qy);
+                src = j - p + (rev_x ? D - 1 - qx : qx) * D + (rev_y ? D - 1 - qy : qy);
             }
             if (j < j1) {
                 wv[u] = w[j];
@@ -1615,7 +1622,9 @@ int run_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
 {
     Timed t(ctx, kClsUpdate);
-    uint32_t parts = (1024 + ctx->N - 1) / ctx->N;
+    // about 1024 blocks; a small SOM (every block repeats the search for the best match) does better with about 128
+    const uint32_t target_blocks = (size_t)ctx->N * ctx->S >= ((size_t)1 << 20) ? 1024u : 128u;
+    uint32_t parts = (target_blocks + ctx->N - 1) / ctx->N;
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
     UpdatePlanes up{};
     if (ctx->fused_som) {
