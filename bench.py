@@ -47,16 +47,16 @@ MEASURED_FMA_NOPACK_TFLOPS = 72.5
 # by what the same counter reads for a device-to-device copy of known size; (bytes, the summary
 # under profiles/ that holds the readings).  Not measured in the run that prints the line.
 COUNTER_TRAFFIC_PER_IMAGE = {
-    ("cfg1", "rotate"): (49.2e3 + 103.8e3, "profiles/cfg1_map_u8_hbm_traffic.txt"),
-    ("cfg1", "distance"): (107.3e3 + 0.8e3, "profiles/cfg1_map_u8_hbm_traffic.txt"),
     ("cfg0", "distance"): (9.641e6 + 0.038e6, "profiles/cfg0_train_f32_counters.txt"),
-    ("cfg0", "update"): (1.436e6 + 1.203e6, "profiles/cfg0_train_f32_counters.txt"),
-    ("cfg2", "distance"): (35.867e6 + 7.078e6 + 5.923e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (25.027e6 + 20.741e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (466.158e6 + 0.307e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg3", "update"): (104.633e6 + 140.110e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg4", "distance"): (0.152e6 + 0.001e6, "profiles/cfg4_train_u8_counters.txt"),
-    ("cfg4", "update"): (0.397e6 + 0.320e6, "profiles/cfg4_train_u8_counters.txt"),
+    ("cfg0", "update"): (1.574e6 + 1.184e6, "profiles/cfg0_train_f32_counters.txt"),
+    ("cfg1", "rotate"): ((96.393e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg1", "distance"): ((214.625e6 + 1.641e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg2", "distance"): (35.856e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (25.055e6 + 20.739e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg3", "distance"): (466.683e6 + 0.307e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "update"): (103.415e6 + 139.967e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg4", "distance"): (0.158e6 + 0.001e6, "profiles/cfg4_train_u8_counters.txt"),
+    ("cfg4", "update"): (0.431e6 + 0.307e6, "profiles/cfg4_train_u8_counters.txt"),
 }
 
 # Images per step of the workloads that ride along in `all_configs` (the headline workload always
