@@ -735,6 +735,121 @@ __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict
     }
 }
 
+// The same distance for large problems (many waves per SIMD): the neuron values are scalar operands.
+// A DPP operand halves the issue rate of the subtract (measured: 5.9 against 3.2 clocks per instruction
+// with eight waves per SIMD), which a lone wave does not notice -- it issues only every other turn anyway --
+// but a full SIMD does.  Here a wave reads its neurons' elements with scalar loads (the neuron is the same
+// for all lanes) and `v_sub_f32 d, s, v` runs at the full rate; stages of 32 elements and few registers
+// let eight blocks share a CU.  Same chains, same order, same results.
+template <int TN, int KC, int MINB, int SW>
+__global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restrict__ somP, const float *__restrict__ rotT,
+                                                           unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
+                                                           uint32_t R, uint32_t Rpad)
+{
+    static_assert(KC == 64 || KC == 32, "stage width");
+    static_assert(SW == 16 || SW == 8, "slab width");
+    constexpr int ROW = KC + 4;
+    constexpr int SLABS = KC / SW;
+    constexpr int VPT = KC / 16;
+    constexpr int TPR = KC / 4;
+    constexpr int RSTEP = 256 / TPR;
+    __shared__ v4f s_rot[2][64 * ROW / 4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t r0 = blockIdx.x * kWave;
+    const uint32_t n0 = blockIdx.y * (4 * TN) + wave * TN;
+    const uint32_t b = blockIdx.z;
+    const float *rp = rotT + ((size_t)b * Rpad + r0) * Epad;
+    const float *np[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad;
+    float acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
+
+    const uint32_t lrow = tid / TPR, lcol = (tid % TPR) * 4;
+    const float *lp = rp + (size_t)lrow * Epad + lcol;
+    const size_t rstep = (size_t)RSTEP * Epad;
+    const uint32_t lds_w = (lrow * ROW + lcol) / 4;
+    const uint32_t lds_wstep = RSTEP * ROW / 4;
+    const uint32_t nchunks = Epad / KC;
+    v4f st[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) s_rot[0][lds_w + i * lds_wstep] = *(const v4f *)(lp + i * rstep);
+    if (nchunks > 1) {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp + KC + i * rstep);
+    }
+    __syncthreads();
+
+    // Operands of a slab of SW elements wait in registers one slab ahead: the lane's SW rotation values
+    // (vector registers, from LDS) and the wave's TN x SW neuron values (scalar registers), in two sets
+    // that take turns.  Slab 0 of a chunk also moves the staged chunk c+1 into the other stage and requests
+    // chunk c+2; the barrier stands before the last slab: by then every wave holds all of chunk c in
+    // registers (its last slab prefetched) and has stored its part of chunk c+1, so the last slab may
+    // prefetch slab 0 of chunk c+1 and the next chunk may overwrite this one's stage.
+    float bv[2][SW];
+    float an[2][TN][SW];
+    auto fetch = [&](int set, uint32_t c, int sl) {
+        const v4f *from = s_rot[c & 1] + lane * (ROW / 4) + sl * (SW / 4);
+#pragma unroll
+        for (int q = 0; q < SW / 4; ++q) {
+            const v4f t4 = from[q];
+            bv[set][4 * q] = t4.x; bv[set][4 * q + 1] = t4.y; bv[set][4 * q + 2] = t4.z; bv[set][4 * q + 3] = t4.w;
+        }
+        const uint32_t k = min(c * KC + sl * SW, Epad - SW);     // (past the end: values nobody uses)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < SW; ++e) an[set][j][e] = np[j][k + e];
+    };
+    fetch(0, 0, 0);
+    for (uint32_t c = 0; c < nchunks; ++c) {
+#pragma unroll
+        for (int sl = 0; sl < SLABS; ++sl) {
+            const int set = sl & 1;
+            // this slab's operands were requested a slab ago; scalar loads return in any order, so the
+            // counter can only be waited down to zero: do it before the next requests join it
+            // (the builtin, not inline assembly: the compiler's own wait insertion must know of it, or it
+            // waits again at the first use, after the new requests; 0xc07f = lgkmcnt(0), the others untouched)
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            if (sl + 1 < SLABS) fetch(set ^ 1, c, sl + 1);
+            else fetch(set ^ 1, c + 1, 0);
+            if (sl == 0) {
+                if (c + 1 < nchunks) {
+                    v4f *nx = s_rot[(c + 1) & 1];
+#pragma unroll
+                    for (int i = 0; i < VPT; ++i) nx[lds_w + i * lds_wstep] = st[i];
+                }
+                if (c + 2 < nchunks) {
+                    const uint32_t k = (c + 2) * KC;
+#pragma unroll
+                    for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp + k + i * rstep);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < SW; ++e)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const float d = __fsub_rn(an[set][j][e], bv[set][e]);
+                    acc[j] = __builtin_fmaf(d, d, acc[j]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+            if (sl == SLABS - 2) __syncthreads();
+        }
+    }
+
+    const uint32_t r = r0 + lane;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | r;
+        if (r >= R) kv = ~0ull;
+        kv = wave_min_u64(kv);
+        if (lane == 0 && n0 + j < N) atomicMin(&key[(size_t)b * N + n0 + j], kv);
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // uint8 distance on the matrix cores (mapping).
 //
@@ -1523,24 +1638,28 @@ void launch_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 // Distance + argmin of B images starting at image slot `slot` of the current launch group.
 void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
-    // Neurons per block = 4 waves x TN: the largest TN that still leaves about four waves per SIMD
-    // (TN = 1 spends as long in LDS reads as in arithmetic, so it is the last resort).
+    // A block is 4 waves x TN neurons x 64 rotations.  While the one-neuron-per-wave blocks are all resident
+    // at once (four per CU; measured up to 225 neurons x 720 rotations): neuron values by DPP broadcast,
+    // deep register prefetch.  More work than that: neuron values as scalar operands, the largest TN that
+    // still leaves the chip about four waves per SIMD (a rotation value read from LDS then serves TN chains).
     const uint32_t rblocks = ctx->Rpad / kWave;
-    uint32_t tn = 4;
-    while (tn > 1 && (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B < (size_t)4 * ctx->num_cu) tn >>= 1;
+    auto blocks = [&](uint32_t tn) { return (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B; };
+    const bool scalar_operands = blocks(1) > (size_t)4 * ctx->num_cu;
+    const uint32_t tn = !scalar_operands ? 1 : blocks(4) >= (size_t)4 * ctx->num_cu ? 4 : 2;
     const dim3 grid(rblocks, (ctx->N + 4 * tn - 1) / (4 * tn), B);
     const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
-#define LAUNCH_TN(...)                                                                                             \
+#define LAUNCH_DPP(...)                                                                                            \
     hipLaunchKernelGGL((k_dist_f32_dpp<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
                        ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
-    // second parameter: chunks of operand prefetch held in registers (deep where waves are few)
-    switch (tn) {
-    case 4: LAUNCH_TN(4, 2, 16); break;
-    case 2: LAUNCH_TN(2, 1, 64); break;
-    default: LAUNCH_TN(1, 2, 64); break;
-    }
-#undef LAUNCH_TN
+#define LAUNCH_SG(...)                                                                                             \
+    hipLaunchKernelGGL((k_dist_f32_sg<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
+                       ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    if (!scalar_operands) LAUNCH_DPP(1, 2, 64);                // (1 neuron per wave, 2 chunks of prefetch, whole-stage LDS batches)
+    else if (tn == 4) LAUNCH_SG(4, 32, 6, 8);                  // 8-element slabs: 4 x 8 x 2 sets of scalar registers
+    else LAUNCH_SG(2, 32, 6, 16);
+#undef LAUNCH_DPP
+#undef LAUNCH_SG
 }
 
 // Distances of B images starting at image slot `slot`.  One image (training): k is cut into

@@ -141,6 +141,38 @@ def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
         assert np.array_equal(best, obest), choice
 
 
+# The float32 distance kernel has two forms chosen by the amount of work per launch: neuron values by DPP
+# broadcast (blocks of one neuron per wave, while they are all resident at once) and neuron values as scalar
+# operands with two or four neurons per wave.  Same chains, same order: every form is bit-equal to the oracle.
+@pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_,n_map", [
+    (397, 1, 64, 44, 360, True, 32, capi.QUADRATIC, 0),      # one image: scalar operands, two neurons per wave
+    (1597, 1, 64, 44, 360, True, 32, capi.QUADRATIC, 0),     # one image: four neurons per wave
+    (70, 1, 20, 14, 32, True, 9, capi.CIRCULAR, 300),        # a launch group of small images: four neurons per wave, two stages
+    (37, 1, 40, 29, 16, True, 21, capi.CIRCULAR, 150),       # ... two neurons per wave, neuron count not a multiple of 8
+])
+def test_float32_distance_forms(N, C_, I, D, nrot, flip, ed, shape_, n_map):
+    say("float32 distance forms", N, C_, I, D, nrot, flip, ed, shape_, n_map)
+    rng = np.random.default_rng(N * 31 + n_map)
+    som = rng.random((N, C_ * D * D), dtype=np.float32)
+    s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, capi.FLOAT)
+    with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, capi.FLOAT) as ctx:
+        ctx.set_som(som)
+        if n_map == 0:
+            img = rng.random((C_, I, I), dtype=np.float32)
+            som[N // 2] = O.rotated_images(img, C_, I, D, nrot, flip)[min(5, nrot - 1)].ravel()   # an exact match
+            ctx.set_som(som)
+            od, _, obest = O.distance_matrix(s, som, O.rotated_images(img, C_, I, D, nrot, flip))
+            d, _, best = ctx.distance(img)
+            assert np.array_equal(bits(d), bits(od))
+            assert np.array_equal(best, obest)
+        else:
+            imgs = rng.random((n_map, C_, I, I), dtype=np.float32)
+            heat, best = ctx.map(imgs)
+            oheat, obest = O.map_images(s, som, imgs)
+            assert np.array_equal(bits(heat), bits(oheat))
+            assert np.array_equal(best, obest)
+
+
 TRAIN_CASES = [
     # workload, images, ed_type override, distance kernel
     ("cfg0", 6, None, capi.KERNEL_AUTO), ("cfg4", 40, None, capi.KERNEL_AUTO), ("cfg4", 10, None, capi.KERNEL_VALU),
