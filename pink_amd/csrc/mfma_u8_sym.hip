@@ -567,34 +567,30 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
     // unit u into `acc`, and a slice of the other work: one (column, row) pair of unit u-1's
     // bookkeeping from `acc_prev` / `cj_prev`, the staging registers (unit u+1) to the next buffer,
     // the barrier, the loads of unit u+2, and this unit's own norm entries for the next round.
-    auto run_unit = [&](uint32_t u, v16i (&acc)[2][2], int (&cj)[16], const v16i (&acc_prev)[2][2], const int (&cj_prev)[16]) {
+    auto run_unit = [&](uint32_t u, v16i (&acc)[2], int (&cj)[16], const v16i (&acc_prev)[2], const int (&cj_prev)[16]) {
         const v4i *cur = s_b + off_cur + lane, *nxt = s_b + off_next + lane;
         v4i *dst = s_b + off_next + tid;
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        // The 32 (column, row) pairs of unit u-1 go through three steps -- sum of the two chains,
-        // shift and add of the norm entry, running maximum -- one pair behind the other: slot s does
-        // the sum of pair s, the shift-add of pair s-1 and the maximum of pair s-2, so that no step
-        // waits for the one before it in the same slot (a lone wave pays about 14 clocks per dependent
-        // vector instruction, and three of them in a row would hold up the next MFMA).
-        uint32_t pair_sum[2], pair_cand[2];
+        // The 32 (column, row) pairs of unit u-1: shift and add of the norm entry, one pair per slot, and
+        // a three-way maximum for every two pairs of a column, two slots behind (a lone wave issues an
+        // instruction only every other turn of its SIMD, so every instruction between two MFMAs counts:
+        // one accumulation chain per column tile and v_max3 keep it at three quarters of an instruction
+        // per MFMA).
+        uint32_t cand[4];
         auto book = [&](int s0, int s1) {
 #pragma unroll
             for (int sl = s0; sl < s1; ++sl) {
-                if (sl >= 2 && sl < 34) {
+                if (sl >= 2 && sl < 34 && (sl & 1) == 0) {
                     const int e = sl - 2, ct = (e >> 2) & 1;
-                    m[ct] = max(m[ct], (int)pair_cand[e & 1]);
-                }
-                if (sl >= 1 && sl < 33) {
-                    const int e = sl - 1, j = 4 * (e >> 3) + (e & 3);
-                    pair_cand[e & 1] = (pair_sum[e & 1] << 5) + (uint32_t)cj_prev[j];
+                    m[ct] = max(max(m[ct], (int)cand[e & 3]), (int)cand[(e + 1) & 3]);
                 }
                 if (sl < 32) {
                     const int e = sl, ct = (e >> 2) & 1, j = 4 * (e >> 3) + (e & 3);
-                    pair_sum[e & 1] = (uint32_t)(acc_prev[ct][0][j] + acc_prev[ct][1][j]);
+                    cand[e & 3] = ((uint32_t)acc_prev[ct][j] << 5) + (uint32_t)cj_prev[j];
                 }
             }
             // pins the slot where it stands
-            asm volatile("" : "+v"(m[0]), "+v"(m[1]), "+v"(pair_sum[0]), "+v"(pair_sum[1]), "+v"(pair_cand[0]), "+v"(pair_cand[1]));
+            asm volatile("" : "+v"(m[0]), "+v"(m[1]), "+v"(cand[0]), "+v"(cand[1]), "+v"(cand[2]), "+v"(cand[3]));
         };
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -604,10 +600,10 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             }
             bf[(ks + 3) & 3] = ks + 3 < KS ? cur[(ks + 3) * 64] : nxt[(ks + 3 - KS) * 64];
-            acc[0][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[0][ks], ks > 1 ? acc[0][ks & 1] : zero, 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[0][ks], ks > 0 ? acc[0] : zero, 0, 0, 0);
             book((2 * ks) * 17 / KS, (2 * ks + 1) * 17 / KS);
             __builtin_amdgcn_sched_barrier(0);
-            acc[1][ks & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[1][ks], ks > 1 ? acc[1][ks & 1] : zero, 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 3], a[1][ks], ks > 0 ? acc[1] : zero, 0, 0, 0);
             book((2 * ks + 1) * 17 / KS, (2 * ks + 2) * 17 / KS);
             // (past the last unit the staging moves data nobody reads: no branches in the k loop)
             if (ks >= W0 && ks < W0 + PER_T) dst[256 * (ks - W0)] = stage[ks - W0];
@@ -630,14 +626,14 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
         off_cur = off_next; off_next = off_free; off_free = o;
     };
 
-    // two accumulator sets (units alternate), each two columns x two chains (even / odd k-steps):
-    // four independent MFMA chains keep the matrix pipe at its issue rate
-    v16i acc0[2][2], acc1[2][2];
+    // two accumulator sets (units alternate), each two columns; the two columns' MFMAs alternate, so a
+    // column's next MFMA finds the one before it finished
+    v16i acc0[2], acc1[2];
     int cj0[16], cj1[16];
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc1[ct][0][j] = acc1[ct][1][j] = 0;
+        for (int j = 0; j < 16; ++j) acc1[ct][j] = 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) cj1[j] = 0;
     for (uint32_t u = 0; u < nunits; u += 2) {
@@ -651,7 +647,7 @@ __global__ __launch_bounds__(256, 1) void k_dist_mfma_sym_u8(const v4i *__restri
         for (int j = 0; j < 16; ++j)
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
-                const int av = (u & 1) ? acc1[ct][0][j] + acc1[ct][1][j] : acc0[ct][0][j] + acc0[ct][1][j];
+                const int av = (u & 1) ? acc1[ct][j] : acc0[ct][j];
                 const int cv = (u & 1) ? cj1[j] : cj0[j];
                 m[ct] = max(m[ct], (int)(((uint32_t)av << 5) + (uint32_t)cv));
             }

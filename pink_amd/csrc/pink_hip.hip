@@ -2588,7 +2588,7 @@ struct StaticPieces {
     size_t per_image() const { return key + Pb + nb + gPb + gnb + rot + rotT; }
 };
 
-StaticPieces static_pieces(const pink_hip_ctx *ctx)
+static StaticPieces static_pieces(const pink_hip_ctx *ctx)
 {
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     StaticPieces p;
