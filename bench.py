@@ -49,12 +49,12 @@ MEASURED_FMA_NOPACK_TFLOPS = 72.5
 COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg0", "distance"): (9.641e6 + 0.038e6, "profiles/cfg0_train_f32_counters.txt"),
     ("cfg0", "update"): (1.574e6 + 1.184e6, "profiles/cfg0_train_f32_counters.txt"),
-    ("cfg1", "rotate"): ((96.393e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg1", "distance"): ((214.625e6 + 1.641e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg2", "distance"): (35.856e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (25.055e6 + 20.739e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (466.683e6 + 0.307e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg3", "update"): (103.415e6 + 139.967e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg1", "rotate"): ((95.060e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg1", "distance"): ((214.633e6 + 1.639e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg2", "distance"): (35.867e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (25.055e6 + 20.737e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg3", "distance"): (674.480e6 + 0.307e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "update"): (103.417e6 + 139.963e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     ("cfg4", "distance"): (0.158e6 + 0.001e6, "profiles/cfg4_train_u8_counters.txt"),
     ("cfg4", "update"): (0.431e6 + 0.307e6, "profiles/cfg4_train_u8_counters.txt"),
 }
