@@ -20,11 +20,15 @@
  *     caller turns into pink::exception;
  *   - a context owns one HIP stream and all its device buffers, shares no global
  *     state with other contexts, and must not be used from two threads at once;
- *   - results follow the reference CPU path: rotated pixels and trained weights
- *     bit-for-bit, float32 distances in the CPU's summation order, integer
- *     (uint8/uint16) distances as exact integer sums of squared differences of
- *     q = T(x * (2^bits - 1)) (CudaLib/copy_and_transform_kernel.h:27-28), lowest
- *     index on ties everywhere.
+ *   - results follow the reference CPU path: rotated pixels and the update arithmetic
+ *     bit-for-bit; float32 distances in the CPU's summation order, one fused
+ *     multiply-add per step where the CPU rounds to double and then to float (the two
+ *     can differ by one unit in the last place of a partial sum, about once in 2^29
+ *     steps; distances therefore agree to 1e-5 relative and are bit-equal in practice,
+ *     trained weights to 1e-4); integer (uint8/uint16) distances as exact integer sums
+ *     of squared differences of q = T(x * (2^bits - 1))
+ *     (CudaLib/copy_and_transform_kernel.h:27-28); lowest index on ties everywhere.
+ *     kernel_choice PINK_HIP_KERNEL_MFMA_F32 alone leaves the CPU's summation order.
  */
 #ifndef PINK_HIP_H
 #define PINK_HIP_H

@@ -4,7 +4,8 @@
 // (src/SelfOrganizingMapLib/Trainer.h:201-335, Mapper.h:129-230).  The kernels are
 // written for CDNA4: 64-lane wavefronts, lanes own rotations so that every global
 // access of the hot loop is a coalesced 256-byte row, neuron values arrive through
-// scalar loads, and the argmin over rotations is a packed 64-bit atomic minimum.
+// DPP broadcasts or scalar loads, and the argmin over rotations is a packed 64-bit
+// atomic minimum.
 //
 // Numerical contract (what the parity tests check against the CPU path):
 //   * rotated pixels: every product and sum rounded separately, in the order of
@@ -12,8 +13,10 @@
 //   * float32 distance: one lane owns one (neuron, rotation) pair and accumulates
 //     fma(d, d, acc) over the region in the CPU's element order
 //     (ImageProcessingLib/euclidean_distance.h:47-100: the CPU squares in double and
-//     rounds the running sum to float at every step, which a fused multiply-add
-//     reproduces);
+//     rounds the running sum to double, then to float, at every step; a fused
+//     multiply-add rounds once, which differs from that by one unit in the last place
+//     about once in 2^29 steps -- within the 1e-5 gate by orders of magnitude, and
+//     bit-equal on the tests' seeds);
 //   * integer distance: exact sums of squared differences of quantised values;
 //   * update: w - ((w - x) * f), three roundings (SelfOrganizingMapLib/Trainer.h:175).
 #include <hip/hip_runtime.h>
