@@ -1237,6 +1237,190 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Small uint8 trainers (at most 64 neurons and 32 variants, e.g. 8 x 8 neurons of 28 x 28 pixels under
+// the eight symmetries): the whole step of an image -- distances, best match, update, operand refresh --
+// in ONE launch.  Two dependent launches cost such a trainer about 5 us each whatever they compute; the
+// distance matrix itself is a few dozen MFMAs.  So every block (one per neuron) computes the WHOLE
+// matrix again (four waves cut k four ways and meet in LDS), finds the best match and its own neuron's
+// best variant, and updates its neuron.  Everything the update needs that does not depend on the search
+// is requested at the start (the neuron's weights, its column of the factor matrix, all stored variants
+// into LDS), so after the search nothing waits for memory.  Blocks run side by side and read all rows of
+// the SOM operand while others rewrite theirs: the operand and its norms therefore alternate between two
+// buffers, every block writing its whole row of the next one (an untouched neuron's row comes out the
+// same bytes).  Arithmetic and tie rules are those of k_dist_gemm_int + k_update.
+// ---------------------------------------------------------------------------------
+struct SmallTrain {
+    const long long *na_cur;
+    long long *na_next;
+    const long long *nb;            // norms of this image's variant rows
+    const uint32_t *variant;        // operand row -> variant index
+    uint32_t *bmu_out, *counts;
+    uint32_t N, S, R, KS, nstored;  // nstored: variants k_rotate stored for this image (two per base rotation)
+    VariantPair vp;
+};
+
+template <int EPT, int KSW>    // elements of a neuron per thread; k-steps per wave held in registers at a time
+__global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som, const float *__restrict__ rot,
+                                                        const v4i *__restrict__ Pa, signed char *__restrict__ Pa_next,
+                                                        const v4i *__restrict__ Pb, const float *__restrict__ factors,
+                                                        const uint32_t *__restrict__ inv, SmallTrain a)
+{
+    extern __shared__ float s_var[];                      // the stored variants of this image
+    __shared__ int s_part[4][2][16][64];                  // [wave][column tile][accumulator][lane]
+    __shared__ unsigned long long s_key[4][32];
+    __shared__ float s_f[64];
+    __shared__ long long s_sq[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = blockIdx.x;
+    const uint32_t N = a.N, S = a.S, KS = a.KS;
+    const bool two = N > 32;
+
+    // (1) Every request that does not depend on the search goes out before anything is waited for, the
+    // operand fragments first (loads return in order: the MFMAs below then wait for them alone).
+    // (no branches here or around the MFMAs: a k-step past the end is loaded from the last one and multiplied
+    // by zeros, a SOM of one column tile multiplies that tile twice)
+    v4i fb[KSW], fa0[KSW], fa1[KSW];
+    const uint32_t tile1 = two ? KS : 0u;
+    auto load_fragments = [&](uint32_t first) {
+#pragma unroll
+        for (int u = 0; u < KSW; ++u) {
+            const uint32_t ks = min(first + 4 * u, KS - 1);
+            fb[u] = Pb[(size_t)ks * 64 + lane];
+            fa0[u] = Pa[(size_t)ks * 64 + lane];
+            fa1[u] = Pa[(size_t)(tile1 + ks) * 64 + lane];
+        }
+    };
+    load_fragments(wave);
+    // this thread's part of the finish: column tile `ct`, eight of the 16 accumulator rows
+    const uint32_t ct = wave & 1, col = lane & 31, m = ct * 32 + col;
+    long long na_m = 0, nb_r[8];
+    uint32_t var_r[8];
+    if (m < N) na_m = a.na_cur[m];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t j = 8 * (wave >> 1) + jj, row = 8 * (j >> 2) + 4 * (lane >> 5) + (j & 3);     // < 32
+        nb_r[jj] = a.nb[row];
+        var_r[jj] = a.variant[row];
+    }
+    float wv[EPT];
+    uint32_t kk[EPT];
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        const uint32_t j = tid + 256 * u;
+        wv[u] = 0.0f; kk[u] = 0xffffffffu;
+        if (j < S) { wv[u] = som[(size_t)n * S + j]; kk[u] = inv[j]; }
+    }
+    const float f_if = tid < N ? factors[(size_t)tid * N + n] : 0.0f;     // the factor, should neuron `tid` be the best match
+    const uint32_t n_var = a.nstored * S;
+    float sv[8];                                          // the first 2048 variant elements wait in registers
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const uint32_t t = tid + 256 * u;
+        sv[u] = t < n_var ? rot[t] : 0.0f;
+    }
+
+    // (2) all dot products: this wave's k-steps, both column tiles
+    v16i acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[t][j] = 0;
+    for (uint32_t first = wave; first < KS; first += 4 * KSW) {
+        if (first != wave) load_fragments(first);
+#pragma unroll
+        for (int u = 0; u < KSW; ++u) {
+            const v4i zero = {0, 0, 0, 0};
+            const v4i b = first + 4 * u < KS ? fb[u] : zero;
+            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa0[u], acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa1[u], acc[1], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s_part[wave][t][j][lane] = acc[t][j];
+    if (tid < 64) s_f[tid] = f_if;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const uint32_t t = tid + 256 * u;
+        if (t < n_var) s_var[t] = sv[u];
+    }
+    for (uint32_t t = tid + 2048; t < n_var; t += 256) s_var[t] = rot[t];
+    __syncthreads();
+
+    // (3) keys: accumulator j of lane l is variant row 8 (j / 4) + 4 (l / 32) + j % 4, neuron column l % 32
+    unsigned long long best = ~0ull;
+    if (m < N) {
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            const uint32_t j = 8 * (wave >> 1) + jj, row = 8 * (j >> 2) + 4 * (lane >> 5) + (j & 3);
+            if (row < a.R) {
+                const long long d = (long long)s_part[0][ct][j][lane] + s_part[1][ct][j][lane] + s_part[2][ct][j][lane] +
+                                    s_part[3][ct][j][lane];
+                const unsigned long long kv = ((unsigned long long)(na_m + nb_r[jj] - 2 * d) << 16) | var_r[jj];
+                best = kv < best ? kv : best;
+            }
+        }
+    }
+    {
+        const unsigned long long o = __shfl_xor(best, 32, 64);
+        best = o < best ? o : best;
+    }
+    if (lane < 32) s_key[wave][lane] = best;
+    __syncthreads();
+    // neuron c's key: the minimum of the two waves that hold its column tile; best match: first minimum of
+    // the distances (Trainer.h:164-168), found by every wave for itself
+    auto key_of = [&](uint32_t c) {
+        const unsigned long long k0 = s_key[c >> 5][c & 31], k1 = s_key[(c >> 5) + 2][c & 31];
+        return k1 < k0 ? k1 : k0;
+    };
+    unsigned long long cand = ~0ull;
+    if (lane < N) cand = ((key_of(lane) >> 16) << 8) | lane;
+    const uint32_t bmu = (uint32_t)(wave_min_u64(cand) & 255u);
+    const uint32_t r = (uint32_t)(key_of(n) & 0xffffu);
+    const float f = s_f[bmu];
+    if (n == 0 && tid == 0) {
+        *a.bmu_out = bmu;
+        atomicAdd(&a.counts[bmu], 1u);                    // m_update_info[bmu]++ (Trainer.h:302-303)
+    }
+
+    // (4) update (Trainer.h:175) and the neuron's row of the next SOM operand
+    const uint32_t D = max(a.vp.D, 1u);
+    const uint32_t flip = r >= a.vp.num_rot ? 1u : 0u, rem = r - flip * a.vp.num_rot;
+    const uint32_t q = rem / a.vp.nrr, i = rem - q * a.vp.nrr;
+    const float *x = s_var + (size_t)((q & 1) * a.vp.nrr + i) * S;
+    const uint32_t rev_x = flip ^ (q >> 1), rev_y = q >> 1;
+    const RcpDivisor by_DD(D * D), by_D(D);
+    long long sq = 0;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        const uint32_t j = tid + 256 * u;
+        if (j < S) {
+            float nv = wv[u];
+            if (f != 0.0f) {
+                uint32_t c, p, qx, qy;
+                by_DD.divmod(j, c, p);
+                by_D.divmod(p, qx, qy);
+                const uint32_t src = j - p + (rev_x ? D - 1 - qx : qx) * D + (rev_y ? D - 1 - qy : qy);
+                nv = __fsub_rn(nv, __fmul_rn(__fsub_rn(nv, x[src]), f));
+                som[(size_t)n * S + j] = nv;
+            }
+            const uint32_t k = kk[u];
+            if (k != 0xffffffffu) {
+                const int h = quantise(nv, 255.0f) - 128;
+                const size_t byte = ((((size_t)(n >> 5) * KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
+                Pa_next[byte] = (signed char)h;
+                sq += h * h;
+            }
+        }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    if (lane == 0) s_sq[wave] = sq;
+    __syncthreads();
+    if (tid == 0) a.na_next[n] = s_sq[0] + s_sq[1] + s_sq[2] + s_sq[3];
+}
+
 // Decode keys: distance (optionally square-rooted for the mapper, Mapper.h:206), exact
 // integer sum, best rotation.  Integer modes: distance = float(double(ssd) / factor^2).
 __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__restrict__ key, float *__restrict__ dist,
@@ -1338,6 +1522,9 @@ struct pink_hip_ctx {
     bool gemm = false;
     uint32_t gKS = 0, Np = 0, Rp = 0, gslices = 1, gks_per = 0;   // k-slices (blocks per tile), k-steps per wave
     v4i *d_gPa = nullptr, *d_gPb = nullptr;
+    v4i *d_gPa_alt = nullptr;             // small uint8 trainers: the SOM operand alternates between two buffers
+    uint32_t pa_cur = 0;                   // ... which of them holds the current SOM
+    bool small_train = false;              // ... one launch per image (k_train_small_u8)
     uint32_t *d_grow = nullptr, *d_gvariant = nullptr;   // variant index -> row of the variant operand, and back
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
@@ -1471,6 +1658,9 @@ bool is_int(const pink_hip_ctx *ctx) { return ctx->cfg.ed_type != PINK_HIP_FLOAT
 
 // --- launch groups ---------------------------------------------------------------
 
+// The SOM operand of the integer GEMM path that holds the current SOM (small uint8 trainers alternate between two).
+static inline v4i *cur_gPa(const pink_hip_ctx *ctx) { return ctx->pa_cur ? ctx->d_gPa_alt : ctx->d_gPa; }
+
 // Matrix-core float32 path: fragments and norms of the SOM rows (after every change of the packed rows).
 int run_pack_frag_som(pink_hip_ctx *ctx)
 {
@@ -1485,10 +1675,10 @@ int run_pack_som(pink_hip_ctx *ctx)
     if (ctx->gemm) {
         if (ctx->cfg.ed_type == PINK_HIP_UINT16)
             hipLaunchKernelGGL(k_pack_planes<true>, dim3(ctx->N, 1), dim3(1024), 2 * ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
+                               cur_gPa(ctx), ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
         else
             hipLaunchKernelGGL(k_pack_planes<false>, dim3(ctx->N, 1), dim3(1024), ctx->gKS * 32, ctx->stream, ctx->d_som, ctx->d_region,
-                               ctx->d_gPa, ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
+                               cur_gPa(ctx), ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, ctx->N, ctx->Np, ctx->S, ctx->E, ctx->gKS, nullptr, PairSource{});
         return launch_check(ctx, "k_pack_planes");
     }
     if (ctx->mfma_sym) {
@@ -1686,7 +1876,7 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
         // a block sees the whole k range: it finishes its tile itself
         fin.key = key; fin.na = na; fin.na_other = na_other; fin.N = ctx->N; fin.R = ctx->R;
     }
-    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, ctx->d_gPa, pb,
+    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
                        (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, slices, tiles_per_xcd, fin);
     if (slices == 1) return;
     const uint32_t rows_per_chunk = 32;
@@ -1750,7 +1940,7 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
     UpdatePlanes up{};
     if (ctx->fused_som) {
-        up.Pa = (signed char *)ctx->d_gPa;
+        up.Pa = (signed char *)cur_gPa(ctx);
         up.na_cur = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np;
         up.na_next = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
         up.KS = ctx->gKS; up.Np = ctx->Np; up.u16 = ctx->cfg.ed_type == PINK_HIP_UINT16;
@@ -1764,6 +1954,35 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
                        is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp);
     if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
+}
+
+// Distances, best match and update of the image in slot `slot` in one launch (small uint8 trainers).
+int run_train_small(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
+{
+    Timed t(ctx, kClsUpdate);
+    SmallTrain a{};
+    a.na_cur = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np;
+    a.na_next = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
+    a.nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
+    a.variant = ctx->d_gvariant;
+    a.bmu_out = dev_bmu_out; a.counts = ctx->d_counts;
+    a.N = ctx->N; a.S = ctx->S; a.R = ctx->R; a.KS = ctx->gKS;
+    a.nstored = std::min(2 * std::max(ctx->nrr, 1u), ctx->R);
+    a.vp.D = ctx->D; a.vp.num_rot = ctx->cfg.num_rot; a.vp.nrr = std::max(ctx->nrr, 1u);
+    const v4i *pa = cur_gPa(ctx);
+    signed char *pa_next = (signed char *)(ctx->pa_cur ? ctx->d_gPa : ctx->d_gPa_alt);
+    const v4i *pb = ctx->d_gPb + (size_t)slot * (ctx->Rp / 32) * ctx->gKS * 64;
+    const float *rot = ctx->d_rot + (size_t)slot * ctx->R * ctx->S;
+    const size_t lds = (size_t)a.nstored * ctx->S * sizeof(float);
+#define LAUNCH_SMALL(...)                                                                                        \
+    hipLaunchKernelGGL((k_train_small_u8<__VA_ARGS__>), dim3(ctx->N), dim3(256), lds, ctx->stream, ctx->d_som, rot, pa, pa_next, pb, \
+                       ctx->d_factors, ctx->d_inv, a)
+    // (elements per thread, k-steps a wave holds at a time: one batch of operand loads up to 32 k-steps)
+    if (ctx->S <= 1024) LAUNCH_SMALL(4, 8); else LAUNCH_SMALL(8, 8);
+#undef LAUNCH_SMALL
+    ctx->pa_cur ^= 1;
+    ctx->na_cur ^= 1;
+    return launch_check(ctx, "k_train_small_u8");
 }
 
 int run_finalize(pink_hip_ctx *ctx, uint32_t B, float *dev_dist, long long *dev_ssd, uint32_t *dev_best, bool do_sqrt)
@@ -1785,7 +2004,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
@@ -2226,6 +2445,16 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipMemcpy(ctx->d_inv, inv.data(), inv.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             ctx->fused_som = ctx->gemm;
         }
+        // one launch per image where the whole distance matrix is a few dozen MFMAs (see k_train_small_u8)
+        const uint32_t nstored = std::min(2 * std::max(ctx->nrr, 1u), ctx->R);
+        ctx->small_train = ctx->fused_som && ctx->pair_variants && c.kernel_choice == PINK_HIP_KERNEL_AUTO &&
+                           c.ed_type == PINK_HIP_UINT8 && ctx->N <= 64 && ctx->R <= 32 && ctx->S <= 2048 && ctx->gKS <= 64 &&
+                           (size_t)nstored * ctx->S * sizeof(float) <= 32768;
+        if (ctx->small_train) {
+            const size_t a_vec = (size_t)(ctx->Np / 32) * ctx->gKS * 64;
+            TRY(dev_alloc(ctx, &ctx->d_gPa_alt, a_vec));
+            HIP_TRY(ctx, hipMemset(ctx->d_gPa_alt, 0, a_vec * sizeof(v4i)));
+        }
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
@@ -2433,6 +2662,10 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
         TRY(run_rotate(ctx, dev_images + (size_t)done * ctx->isz, B, ctx->pair_variants ? kStorePair : kStoreAll));
         TRY(run_pack_rot(ctx, B));
         for (uint32_t b = 0; b < B; ++b) {
+            if (ctx->small_train) {
+                TRY(run_train_small(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
+                continue;
+            }
             TRY(run_dist(ctx, b, 1));
             TRY(run_update(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
             if (!ctx->d_inv || (ctx->gemm && !ctx->fused_som)) TRY(run_pack_som(ctx));
