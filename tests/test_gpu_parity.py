@@ -643,14 +643,19 @@ def test_mfma_kernel_refused_where_it_does_not_apply():
         capi.Context(16, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.FLOAT, kernel_choice=capi.KERNEL_MFMA)
 
 
-def test_profiling_counts_launches():
-    w = synthetic.WORKLOADS["cfg4"]
-    with synthetic.make_context(w) as ctx:
+@pytest.mark.parametrize("name,choice,distance_launches", [
+    ("cfg0", capi.KERNEL_AUTO, 5),
+    ("cfg4", capi.KERNEL_MFMA_GEMM, 5),
+    ("cfg4", capi.KERNEL_AUTO, 0),          # a small uint8 trainer: distance, best match and update in one launch per image
+])
+def test_profiling_counts_launches(name, choice, distance_launches):
+    w = synthetic.WORKLOADS[name]
+    with synthetic.make_context(w, kernel_choice=choice) as ctx:
         ctx.set_som(synthetic.initial_som(w))
         ctx.set_profiling(True)
         ctx.train(synthetic.images(w, 5))
         t = ctx.kernel_times()
         ctx.set_profiling(False)
     # variants are prepared for a group of images per launch; distance and update run per image
-    assert t["rotate"][0] == 1 and t["distance"][0] == 5 and t["update"][0] == 5
+    assert t["rotate"][0] == 1 and t["distance"][0] == distance_launches and t["update"][0] == 5
     assert all(ms >= 0 for _, ms in t.values())
