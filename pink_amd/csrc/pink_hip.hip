@@ -1077,6 +1077,7 @@ struct UpdatePlanes {
     uint32_t KS, Np, u16;
 };
 
+template <uint32_t U>     // elements per thread and round: all their loads are issued before the first store
 __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const float *__restrict__ rot,
                                                 const unsigned long long *__restrict__ key,
                                                 const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
@@ -1092,7 +1093,6 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     // What the block will read does not depend on the best-matching neuron, only whether it is
     // needed does: the first round of loads is issued ahead of the search, which then runs while
     // they are in flight (a neuron with factor 0 drops them).
-    constexpr uint32_t U = 4;
     // (loads return in issue order: the keys go first, so the search below waits for them alone)
     unsigned long long bv = ~0ull;
     uint32_t bi = 0xffffffffu;
@@ -1956,11 +1956,16 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     }
     VariantPair vp{};
     if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
-    hipLaunchKernelGGL(k_update, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
-                       ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors,
-                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,
-                       (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,
-                       is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp);
+#define LAUNCH_UPDATE(U_)                                                                                        \
+    hipLaunchKernelGGL(k_update<U_>, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,                   \
+                       ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors, \
+                       dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,                                \
+                       (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,                           \
+                       is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp)
+    // a slice of several rounds keeps eight elements per thread in flight (cfg2 -6 %, cfg3 -3 % against four);
+    // a slice of one round is faster with four (cfg0 +8 % with eight)
+    if ((ctx->S + parts - 1) / parts > 1024) LAUNCH_UPDATE(8); else LAUNCH_UPDATE(4);
+#undef LAUNCH_UPDATE
     if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
 }
