@@ -744,7 +744,7 @@ __global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict
 // but a full SIMD does.  Here a wave reads its neurons' elements with scalar loads (the neuron is the same
 // for all lanes) and `v_sub_f32 d, s, v` runs at the full rate; stages of 32 elements and few registers
 // let eight blocks share a CU.  Same chains, same order, same results.
-template <int TN, int KC, int MINB, int SW>
+template <int TN, int KC, int MINB, int SW, bool NL>
 __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                            unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
                                                            uint32_t R, uint32_t Rpad)
@@ -759,29 +759,36 @@ __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restri
     __shared__ v4f s_rot[2][64 * ROW / 4];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t r0 = blockIdx.x * kWave;
-    const uint32_t n0 = blockIdx.y * (4 * TN) + wave * TN;
     const uint32_t b = blockIdx.z;
-    const float *rp = rotT + ((size_t)b * Rpad + r0) * Epad;
+    // Rows on the lanes (64 per block, through LDS) and rows as scalar operands (TN per wave): rotations and
+    // neurons, or (NL) neurons and rotations -- whichever wastes fewer lanes on padding.  A chain is the same
+    // sequence of operations either way (the difference changes sign, its square does not).
+    const uint32_t l0 = blockIdx.x * kWave;
+    const uint32_t s0 = blockIdx.y * (4 * TN) + wave * TN;
+    const float *laneP = NL ? somP : rotT + (size_t)b * Rpad * Epad;
+    const float *scalP = NL ? rotT + (size_t)b * Rpad * Epad : somP;
+    const uint32_t lane_rows = NL ? N : Rpad;             // rows that exist on the lane side (loads are clamped to them)
+    const uint32_t scal_rows = NL ? R : N;
     const float *np[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad;
+    for (int j = 0; j < TN; ++j) np[j] = scalP + (size_t)min(s0 + j, scal_rows - 1) * Epad;
     float acc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
 
     const uint32_t lrow = tid / TPR, lcol = (tid % TPR) * 4;
-    const float *lp = rp + (size_t)lrow * Epad + lcol;
-    const size_t rstep = (size_t)RSTEP * Epad;
+    const float *lp[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) lp[i] = laneP + (size_t)min(l0 + lrow + RSTEP * i, lane_rows - 1) * Epad + lcol;
     const uint32_t lds_w = (lrow * ROW + lcol) / 4;
     const uint32_t lds_wstep = RSTEP * ROW / 4;
     const uint32_t nchunks = Epad / KC;
     v4f st[VPT];
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) s_rot[0][lds_w + i * lds_wstep] = *(const v4f *)(lp + i * rstep);
+    for (int i = 0; i < VPT; ++i) s_rot[0][lds_w + i * lds_wstep] = *(const v4f *)(lp[i]);
     if (nchunks > 1) {
 #pragma unroll
-        for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp + KC + i * rstep);
+        for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp[i] + KC);
     }
     __syncthreads();
 
@@ -827,7 +834,7 @@ __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restri
                 if (c + 2 < nchunks) {
                     const uint32_t k = (c + 2) * KC;
 #pragma unroll
-                    for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp + k + i * rstep);
+                    for (int i = 0; i < VPT; ++i) st[i] = *(const v4f *)(lp[i] + k);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -835,7 +842,7 @@ __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restri
             for (int e = 0; e < SW; ++e)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
-                    const float d = __fsub_rn(an[set][j][e], bv[set][e]);
+                    const float d = NL ? __fsub_rn(bv[set][e], an[set][j][e]) : __fsub_rn(an[set][j][e], bv[set][e]);
                     acc[j] = __builtin_fmaf(d, d, acc[j]);
                 }
             __builtin_amdgcn_sched_barrier(0);
@@ -843,13 +850,31 @@ __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restri
         }
     }
 
-    const uint32_t r = r0 + lane;
+    if constexpr (!NL) {
+        const uint32_t r = l0 + lane;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | r;
-        if (r >= R) kv = ~0ull;
-        kv = wave_min_u64(kv);
-        if (lane == 0 && n0 + j < N) atomicMin(&key[(size_t)b * N + n0 + j], kv);
+        for (int j = 0; j < TN; ++j) {
+            unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | r;
+            if (r >= R) kv = ~0ull;
+            kv = wave_min_u64(kv);
+            if (lane == 0 && s0 + j < N) atomicMin(&key[(size_t)b * N + s0 + j], kv);
+        }
+    } else {
+        // a lane is a neuron: the minimum over this wave's TN rotations in the lane, over the block's four waves in LDS
+        __shared__ unsigned long long s_best[4][64];
+        unsigned long long best = ~0ull;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | (s0 + j);
+            if (s0 + j < R && kv < best) best = kv;
+        }
+        s_best[wave][lane] = best;
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int w = 1; w < 4; ++w) best = s_best[w][lane] < best ? s_best[w][lane] : best;
+            if (l0 + lane < N) atomicMin(&key[(size_t)b * N + l0 + lane], best);
+        }
     }
 }
 
@@ -1831,27 +1856,35 @@ void launch_dist(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 // Distance + argmin of B images starting at image slot `slot` of the current launch group.
 void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
-    // A block is 4 waves x TN neurons x 64 rotations.  While the one-neuron-per-wave blocks are all resident
-    // at once (four per CU; measured up to 225 neurons x 720 rotations): neuron values by DPP broadcast,
-    // deep register prefetch.  More work than that: neuron values as scalar operands, the largest TN that
-    // still leaves the chip about four waves per SIMD (a rotation value read from LDS then serves TN chains).
-    const uint32_t rblocks = ctx->Rpad / kWave;
-    auto blocks = [&](uint32_t tn) { return (size_t)rblocks * ((ctx->N + 4 * tn - 1) / (4 * tn)) * B; };
-    const bool scalar_operands = blocks(1) > (size_t)4 * ctx->num_cu;
-    const uint32_t tn = !scalar_operands ? 1 : blocks(4) >= (size_t)4 * ctx->num_cu ? 4 : 2;
-    const dim3 grid(rblocks, (ctx->N + 4 * tn - 1) / (4 * tn), B);
+    // A block is 64 rows on its lanes x (4 waves x TN) rows as per-wave operands.  While the blocks of one
+    // neuron per wave are all resident at once (four per CU; measured up to 225 neurons x 720 rotations):
+    // rotations on the lanes, neuron values by DPP broadcast, deep register prefetch.  More work than that:
+    // per-wave operands as scalar registers, the largest TN that still leaves the chip about four waves per
+    // SIMD (a value read from LDS then serves TN chains), and on the lanes whichever of rotations and neurons
+    // loses fewer lanes to padding (360 rotations fill 5.6 tiles of 64, 1600 neurons exactly 25).
+    const uint32_t rblocks = ctx->Rpad / kWave, nblocks = (ctx->N + kWave - 1) / kWave;
+    auto groups = [](uint32_t rows, uint32_t tn) { return (rows + 4 * tn - 1) / (4 * tn); };
+    const bool scalar_operands = (size_t)rblocks * groups(ctx->N, 1) * B > (size_t)4 * ctx->num_cu;
     const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
-#define LAUNCH_DPP(...)                                                                                            \
-    hipLaunchKernelGGL((k_dist_f32_dpp<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
-                       ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    if (!scalar_operands) {
+        // (1 neuron per wave, 2 chunks of prefetch, whole-stage LDS batches)
+        hipLaunchKernelGGL((k_dist_f32_dpp<1, 2, 64>), dim3(rblocks, groups(ctx->N, 1), B), dim3(256), 0, ctx->stream,
+                           (const float *)ctx->d_somP, rotT, key, ctx->N, ctx->Epad, ctx->R, ctx->Rpad);
+        return;
+    }
+    // lanes computed, padding included, per image: rotations on the lanes / neurons on the lanes (TN = 2 for the comparison)
+    const size_t work_rot = (size_t)rblocks * kWave * groups(ctx->N, 2) * 8, work_neu = (size_t)nblocks * kWave * groups(ctx->R, 2) * 8;
+    const bool neurons_on_lanes = work_neu * 100 < work_rot * 98;
+    const uint32_t lane_blocks = neurons_on_lanes ? nblocks : rblocks, scal_rows = neurons_on_lanes ? ctx->R : ctx->N;
+    const uint32_t tn = (size_t)lane_blocks * groups(scal_rows, 4) * B >= (size_t)4 * ctx->num_cu ? 4 : 2;
+    const dim3 grid(lane_blocks, groups(scal_rows, tn), B);
 #define LAUNCH_SG(...)                                                                                             \
-    hipLaunchKernelGGL((k_dist_f32_sg<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP, rotT, key, \
-                       ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
-    if (!scalar_operands) LAUNCH_DPP(1, 2, 64);                // (1 neuron per wave, 2 chunks of prefetch, whole-stage LDS batches)
-    else if (tn == 4) LAUNCH_SG(4, 32, 6, 8);                  // 8-element slabs: 4 x 8 x 2 sets of scalar registers
-    else LAUNCH_SG(2, 32, 6, 16);
-#undef LAUNCH_DPP
+    hipLaunchKernelGGL((k_dist_f32_sg<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP,  \
+                       (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad, key, ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+    // (TN = 4: 8-element slabs, 4 x 8 x 2 sets of scalar registers)
+    if (neurons_on_lanes) { if (tn == 4) LAUNCH_SG(4, 32, 6, 8, true); else LAUNCH_SG(2, 32, 6, 16, true); }
+    else { if (tn == 4) LAUNCH_SG(4, 32, 6, 8, false); else LAUNCH_SG(2, 32, 6, 16, false); }
 #undef LAUNCH_SG
 }
 
