@@ -130,11 +130,14 @@ int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som);
  * image k, Pink/main_generic.h:87-89); n_images = 1 is exactly one operator() call.
  * bmu_out receives the best-matching neuron of each image, which the caller adds to
  * m_update_info (Trainer.h:302-303); the call then returns when they are there.
- * With bmu_out NULL and up to 128 KiB of images the call copies the images and returns
- * with the work queued on the context's stream (operator() returns nothing either): a
- * loop of per-image calls then runs at the rate of the kernels, not of the round trips.
- * pink_hip_get_som, pink_hip_update_counts and pink_hip_synchronize wait for queued work;
- * an error of queued work is reported by the next call that waits. */
+ * With bmu_out NULL and up to 128 KiB of images the call only copies the images into a
+ * pinned buffer and returns (operator() returns nothing either); they are trained, in
+ * order, a launch group (up to 64 images) at a time: when the group is full or when any
+ * other call on the context follows.  A loop of per-image calls then runs at the rate of
+ * the kernels (the rotation of a group is one launch), not of per-image launches and
+ * round trips, and leaves the weights of training call by call.  pink_hip_get_som,
+ * pink_hip_update_counts and pink_hip_synchronize wait for that work; an error in it is
+ * reported by the call that starts or waits for it. */
 int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images, uint32_t *host_bmu_out);
 /* m_update_info (Trainer.h:79,94-95,302-303): how often each of the N neurons was the
  * best match, over all images this context has trained, counted on the device. */

@@ -1524,6 +1524,10 @@ struct pink_hip_ctx {
     hipEvent_t st_ev[8] = {};              // per slot: the copy out of it has run
     uint32_t st_slot = 0;
     bool st_ring_busy = false;             // a call returned with copies out of the ring still queued
+    // per-image training calls that hand nothing back wait here until a launch group is full (or any other call comes)
+    char *pend_pin[2] = {nullptr, nullptr};
+    hipEvent_t pend_ev[2] = {nullptr, nullptr};
+    uint32_t pend_count = 0, pend_cur = 0, pend_cap = 0;
     hipStream_t copy_stream = nullptr;     // host -> device copies of the next images while the kernels of the last run
     hipEvent_t copy_ev[2] = {};
     uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
@@ -2055,6 +2059,10 @@ int free_all(pink_hip_ctx *ctx)
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
+    for (int i = 0; i < 2; ++i) {
+        if (ctx->pend_pin[i]) (void)hipHostFree(ctx->pend_pin[i]);
+        if (ctx->pend_ev[i]) (void)hipEventDestroy(ctx->pend_ev[i]);
+    }
     for (hipEvent_t e : ctx->st_ev) if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : ctx->copy_ev) if (e) (void)hipEventDestroy(e);
     if (ctx->copy_stream) (void)hipStreamDestroy(ctx->copy_stream);
@@ -2658,9 +2666,29 @@ void pink_hip_destroy(pink_hip_ctx *ctx)
     delete ctx;
 }
 
+// Training calls without a result (the reference's Trainer::operator() returns nothing) only copy their
+// image into a pinned buffer; the images go to the device, and through rotation, distance and update, a
+// launch group at a time: when the group is full, or when any other call on the context needs the state
+// they produce.  The order of the images and every result are those of training them call by call.
+int ensure_staging(pink_hip_ctx *ctx, size_t n);
+int flush_pending(pink_hip_ctx *ctx)
+{
+    if (!ctx || !ctx->pend_count) return PINK_HIP_OK;
+    const uint32_t n = ctx->pend_count, cur = ctx->pend_cur;
+    ctx->pend_count = 0;
+    ctx->pend_cur ^= 1;
+    HIP_TRY(ctx, hipSetDevice(ctx->device));
+    TRY(ensure_staging(ctx, std::max<size_t>(n, ctx->pend_cap)));
+    HIP_TRY(ctx, hipMemcpyAsync(ctx->st_img, ctx->pend_pin[cur], (size_t)n * ctx->isz * sizeof(float), hipMemcpyHostToDevice,
+                                ctx->stream));
+    HIP_TRY(ctx, hipEventRecord(ctx->pend_ev[cur], ctx->stream));
+    return pink_hip_train_device(ctx, ctx->st_img, n, ctx->st_bmu);
+}
+
 int pink_hip_synchronize(pink_hip_ctx *ctx)
 {
     if (!ctx) return PINK_HIP_EINVAL;
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     return PINK_HIP_OK;
@@ -2669,6 +2697,7 @@ int pink_hip_synchronize(pink_hip_ctx *ctx)
 int pink_hip_set_som(pink_hip_ctx *ctx, const float *host_som)
 {
     if (!ctx || !host_som) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_set_som: null argument");
+    TRY(flush_pending(ctx));                              // images trained before this call see the SOM before it
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipMemcpyAsync(ctx->d_som, host_som, (size_t)ctx->N * ctx->S * sizeof(float), hipMemcpyHostToDevice,
                                 ctx->stream));
@@ -2680,6 +2709,7 @@ int pink_hip_set_som(pink_hip_ctx *ctx, const float *host_som)
 int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som)
 {
     if (!ctx || !host_som) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_get_som: null argument");
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipMemcpyAsync(host_som, ctx->d_som, (size_t)ctx->N * ctx->S * sizeof(float), hipMemcpyDeviceToHost,
                                 ctx->stream));
@@ -2691,6 +2721,7 @@ int pink_hip_update_counts(pink_hip_ctx *ctx, uint32_t *host_counts_out)
 {
     if (!ctx || !host_counts_out) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_update_counts: null argument");
     if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_update_counts: context was created without update factors");
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     HIP_TRY(ctx, hipMemcpyAsync(host_counts_out, ctx->d_counts, (size_t)ctx->N * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -2701,6 +2732,7 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
 {
     if (!ctx || (!dev_images && n_images)) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_train_device: null argument");
     if (!ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_train: context was created without update factors");
+    TRY(flush_pending(ctx));                              // (none while flush_pending itself calls this)
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     // The variants of an image and their packed distance operand do not depend on the SOM: they
     // are produced for a group of images per launch.  Distance and update stay strictly sequential.
@@ -2812,20 +2844,31 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     const size_t img_bytes = (size_t)ctx->isz * sizeof(float);
     if (!host_bmu_out && n_images * img_bytes <= kSlotBytes) {
-        // Nothing to hand back (the reference's operator() returns nothing either): the images are
-        // copied into a slot of the pinned ring and the call returns with the work queued, so a loop of
-        // per-image calls keeps the GPU busy instead of waiting for each image in turn.
-        TRY(ensure_staging(ctx, n_images));
-        const uint32_t slot = ctx->st_slot;
-        ctx->st_slot = (slot + 1) % kPinSlots;
-        HIP_TRY(ctx, hipEventSynchronize(ctx->st_ev[slot]));          // the copy that last used the slot has run
-        char *pin = ctx->st_pin + (size_t)slot * kSlotBytes;
-        memcpy(pin, host_images, n_images * img_bytes);
-        HIP_TRY(ctx, hipMemcpyAsync(ctx->st_img, pin, n_images * img_bytes, hipMemcpyHostToDevice, ctx->stream));
-        HIP_TRY(ctx, hipEventRecord(ctx->st_ev[slot], ctx->stream));
-        ctx->st_ring_busy = true;
-        return pink_hip_train_device(ctx, ctx->st_img, n_images, ctx->st_bmu);
+        // Nothing to hand back (the reference's operator() returns nothing either): the images join the
+        // pending launch group in pinned memory and the call returns; see flush_pending.
+        if (!ctx->pend_pin[0]) {
+            ctx->pend_cap = ctx->Bcap;
+            for (int i = 0; i < 2; ++i) {
+                if (hipHostMalloc((void **)&ctx->pend_pin[i], (size_t)ctx->pend_cap * img_bytes, hipHostMallocDefault) != hipSuccess) {
+                    ctx->pend_pin[i] = nullptr;
+                    if (i == 1) { (void)hipHostFree(ctx->pend_pin[0]); ctx->pend_pin[0] = nullptr; }
+                    return fail(ctx, PINK_HIP_ENOMEM, "pinned host allocation failed");
+                }
+                HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->pend_ev[i], hipEventDisableTiming));
+            }
+        }
+        for (uint32_t done = 0; done < n_images;) {
+            const uint32_t take = std::min(n_images - done, ctx->pend_cap - ctx->pend_count);
+            if (ctx->pend_count == 0) HIP_TRY(ctx, hipEventSynchronize(ctx->pend_ev[ctx->pend_cur]));   // its last copy has run
+            memcpy(ctx->pend_pin[ctx->pend_cur] + (size_t)ctx->pend_count * img_bytes, host_images + (size_t)done * ctx->isz,
+                   (size_t)take * img_bytes);
+            ctx->pend_count += take;
+            done += take;
+            if (ctx->pend_count == ctx->pend_cap) TRY(flush_pending(ctx));
+        }
+        return PINK_HIP_OK;
     }
+    TRY(flush_pending(ctx));
     // Stage the images in chunks of at most ~1 GiB.
     const uint32_t chunk = (uint32_t)std::max<size_t>(1, std::min<size_t>(n_images, ((size_t)1 << 30) / img_bytes));
     TRY(ensure_staging(ctx, chunk));
@@ -2990,6 +3033,7 @@ int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
 int pink_hip_rotate(pink_hip_ctx *ctx, const float *host_image, float *host_variants_out)
 {
     if (!ctx || !host_image || !host_variants_out) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_rotate: null argument");
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     float *d_img = nullptr;
     HIP_TRY(ctx, hipMalloc((void **)&d_img, (size_t)ctx->isz * sizeof(float)));
@@ -3009,6 +3053,7 @@ int pink_hip_distance(pink_hip_ctx *ctx, const float *host_image, float *host_di
                       uint32_t *host_best_rot_out)
 {
     if (!ctx || !host_image) return fail(ctx, PINK_HIP_EINVAL, "pink_hip_distance: null argument");
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     float *d_img = nullptr;
     HIP_TRY(ctx, hipMalloc((void **)&d_img, (size_t)ctx->isz * sizeof(float)));
@@ -3041,6 +3086,7 @@ uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx)
 int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)
 {
     if (!ctx) return PINK_HIP_EINVAL;
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     TRY(drain_events(ctx));
     ctx->profiling = enable != 0;
@@ -3051,6 +3097,7 @@ int pink_hip_set_profiling(pink_hip_ctx *ctx, int enable)
 int pink_hip_kernel_times(pink_hip_ctx *ctx, uint64_t *launches_out, double *ms_out)
 {
     if (!ctx) return PINK_HIP_EINVAL;
+    TRY(flush_pending(ctx));
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     TRY(drain_events(ctx));
     for (int i = 0; i < PINK_HIP_NUM_KERNEL_CLASSES; ++i) {
