@@ -218,6 +218,43 @@ def test_train_one_call_per_image_equals_batched_call():
         assert np.array_equal(bits(a.get_som()), bits(b.get_som()))
 
 
+@pytest.mark.parametrize("name,n", [("cfg0", 150), ("cfg4", 200)])
+def test_calls_without_a_result_train_in_order_whatever_comes_between(name, n):
+    """Calls that hand nothing back (the reference's Trainer::operator()) are collected into launch groups;
+    every other call on the context first trains what is pending.  Weights, best matches and counts are those of
+    one call over all images, and of the CPU."""
+    w = synthetic.WORKLOADS[name]
+    imgs = synthetic.images(w, n)
+    som0 = synthetic.initial_som(w)
+    F = synthetic.update_factors(w)
+    s = O.shape(w.som_size, w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip, w.ed_dim, w.ed_shape, w.ed_type)
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(som0)
+        bmu_mid = None
+        for i in range(n):
+            if i == 70:
+                d_mid = ctx.distance(imgs[0])[0]          # sees the SOM after 70 images
+            if i == 100:
+                bmu_mid = ctx.train(imgs[100:103])         # a call with a result, in the middle of pending ones
+                continue
+            if i in (101, 102):
+                continue
+            if i == 120:
+                ctx.rotate(imgs[5])                        # the debug tap shares buffers with the trainer
+            ctx.train(imgs[i], want_bmu=False)             # three of them in one call further down
+        counts = ctx.update_counts()
+        got = ctx.get_som()
+    want = som0.copy()
+    obmu = O.train(s, want, imgs, F)
+    assert np.array_equal(bits(got), bits(want))
+    assert np.array_equal(bmu_mid, obmu[100:103])
+    assert np.array_equal(counts, np.bincount(obmu, minlength=w.som_size))
+    mid = som0.copy()
+    O.train(s, mid, imgs[:70], F)
+    od = O.distance_matrix(s, mid, O.rotated_images(imgs[0], w.channels, w.image_dim, w.neuron_dim, w.num_rot, w.use_flip))[0]
+    assert np.array_equal(bits(d_mid), bits(od))
+
+
 @pytest.mark.parametrize("name", ["cfg4", "cfg0"])
 def test_rotation_tap_between_training_calls(name):
     # a trainer keeps two of a base rotation's eight symmetries; the tap asks for all of them in between
