@@ -41,7 +41,7 @@ DTYPE_NAME = {0: "f32", 1: "u16", 2: "u8"}
 # streams on all CUs): the clock settles near 2.0-2.2 GHz under load.  Reported next to the
 # published figures, never instead of them.
 MEASURED_INT8_MFMA_TOPS = 4130.0
-MEASURED_FMA_NOPACK_TFLOPS = 72.5
+MEASURED_VALU_LANE_OPS_T = 50.0     # subtract / fma stream, eight waves per SIMD: 3.15 clk per wave instruction at 2.4 GHz
 
 # HBM bytes per image of one kernel class from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
 # by what the same counter reads for a device-to-device copy of known size; (bytes, the summary
@@ -250,9 +250,9 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
         bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
         notes = ("compute bound on the vector ALU: bit-faithful sequential fma per (neuron, rotation), one subtract + "
-                 "one fma per pair element (counted as 2 operations), which caps this form at a quarter of the published "
-                 "157.3 TFLOP/s with packed FP32 disabled in this build (measured fma rate %.1f TFLOP/s)"
-                 % MEASURED_FMA_NOPACK_TFLOPS)
+                 "one fma per pair element (counted as 2 operations); non-packed instructions (packed FP32 is disabled in "
+                 "this build) issue at 3.15 clocks per wave at best, measured: %.0f T operations/s = about a third of the "
+                 "published 157.3 TFLOP/s is this form's ceiling" % MEASURED_VALU_LANE_OPS_T)
     elif dominant == "distance" and path in (capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA_GEMM, capi.KERNEL_MFMA):
         bound, unit, peak = "mfma", "TOP/s", MFMA_INT8_PEAK_TOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
