@@ -1285,17 +1285,25 @@ struct SmallTrain {
     VariantPair vp;
 };
 
+// Per neuron element j, prepared once per context (no divisions in the kernel):
+//   src4[j]  = where element j of a variant sits in the stored one, for rows / columns read as stored or reversed:
+//              16 bits for each of the four combinations (rows reversed) * 2 + (columns reversed);
+//   kbyte[j] = byte of element j inside a row of 32-row fragments of the SOM operand, (k / 32) * 1024 +
+//              (k / 16 % 2) * 512 + k % 16 for region position k, or all ones outside the region.
 template <int EPT, int KSW>    // elements of a neuron per thread; k-steps per wave held in registers at a time
 __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som, const float *__restrict__ rot,
                                                         const v4i *__restrict__ Pa, signed char *__restrict__ Pa_next,
                                                         const v4i *__restrict__ Pb, const float *__restrict__ factors,
-                                                        const uint32_t *__restrict__ inv, SmallTrain a)
+                                                        const unsigned long long *__restrict__ src4,
+                                                        const uint32_t *__restrict__ kbyte, SmallTrain a)
 {
     extern __shared__ float s_var[];                      // the stored variants of this image
-    __shared__ int s_part[4][2][16][64];                  // [wave][column tile][accumulator][lane]
-    __shared__ unsigned long long s_key[4][32];
+    // [wave][column tile][lane][16 accumulators + 4]: a lane's accumulators in one place (16-byte accesses), lanes
+    // 80 bytes apart (sixteen neighbouring lanes then cover every bank once)
+    __shared__ v4i s_part[4][2][64][5];
+    __shared__ uint32_t s_key[4][32];
     __shared__ float s_f[64];
-    __shared__ long long s_sq[4];
+    __shared__ int s_sq[4];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = blockIdx.x;
     const uint32_t N = a.N, S = a.S, KS = a.KS;
     const bool two = N > 32;
@@ -1316,54 +1324,53 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
         }
     };
     load_fragments(wave);
-    // this thread's part of the finish: column tile `ct`, eight of the 16 accumulator rows
+    // This thread's part of the finish: column tile `ct`, eight of the 16 accumulator rows.  Sums stay below
+    // 2^27 (at most 2048 elements of 8 bits) and variants below 32: keys are 32 bits, distance * 32 + variant.
     const uint32_t ct = wave & 1, col = lane & 31, m = ct * 32 + col;
-    long long na_m = 0, nb_r[8];
+    int na_m = 0, nb_r[8];
     uint32_t var_r[8];
-    if (m < N) na_m = a.na_cur[m];
+    if (m < N) na_m = (int)a.na_cur[m];
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
         const uint32_t j = 8 * (wave >> 1) + jj, row = 8 * (j >> 2) + 4 * (lane >> 5) + (j & 3);     // < 32
-        nb_r[jj] = a.nb[row];
+        nb_r[jj] = (int)a.nb[row];
         var_r[jj] = a.variant[row];
     }
     float wv[EPT];
-    uint32_t kk[EPT];
+    uint32_t kb[EPT];
+    unsigned long long sp[EPT];
 #pragma unroll
     for (int u = 0; u < EPT; ++u) {
-        const uint32_t j = tid + 256 * u;
-        wv[u] = 0.0f; kk[u] = 0xffffffffu;
-        if (j < S) { wv[u] = som[(size_t)n * S + j]; kk[u] = inv[j]; }
+        const uint32_t j = min(tid + 256 * u, S - 1);     // (past the end: the last element again, dropped below)
+        wv[u] = som[(size_t)n * S + j];
+        kb[u] = kbyte[j];
+        sp[u] = src4[j];
     }
     const float f_if = tid < N ? factors[(size_t)tid * N + n] : 0.0f;     // the factor, should neuron `tid` be the best match
     const uint32_t n_var = a.nstored * S;
     float sv[8];                                          // the first 2048 variant elements wait in registers
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-        const uint32_t t = tid + 256 * u;
-        sv[u] = t < n_var ? rot[t] : 0.0f;
-    }
+    for (int u = 0; u < 8; ++u) sv[u] = rot[min(tid + 256 * u, n_var - 1)];
 
     // (2) all dot products: this wave's k-steps, both column tiles
     v16i acc[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[t][j] = 0;
     for (uint32_t first = wave; first < KS; first += 4 * KSW) {
-        if (first != wave) load_fragments(first);
+        const bool again = first != wave;
+        if (again) load_fragments(first);
 #pragma unroll
         for (int u = 0; u < KSW; ++u) {
             const v4i zero = {0, 0, 0, 0};
+            const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             const v4i b = first + 4 * u < KS ? fb[u] : zero;
-            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa0[u], acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa1[u], acc[1], 0, 0, 0);
+            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa0[u], (u == 0 && !again) ? zero16 : acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, fa1[u], (u == 0 && !again) ? zero16 : acc[1], 0, 0, 0);
         }
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) s_part[wave][t][j][lane] = acc[t][j];
+        for (int g = 0; g < 4; ++g)
+            s_part[wave][t][lane][g] = (v4i){acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
     if (tid < 64) s_f[tid] = f_if;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -1374,35 +1381,34 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
     __syncthreads();
 
     // (3) keys: accumulator j of lane l is variant row 8 (j / 4) + 4 (l / 32) + j % 4, neuron column l % 32
-    unsigned long long best = ~0ull;
-    if (m < N) {
+    uint32_t best = 0xffffffffu;
+    {
+        int dot[8];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            v4i t4 = s_part[0][ct][lane][2 * (wave >> 1) + h];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) t4 += s_part[w][ct][lane][2 * (wave >> 1) + h];
+            dot[4 * h] = t4.x; dot[4 * h + 1] = t4.y; dot[4 * h + 2] = t4.z; dot[4 * h + 3] = t4.w;
+        }
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) {
             const uint32_t j = 8 * (wave >> 1) + jj, row = 8 * (j >> 2) + 4 * (lane >> 5) + (j & 3);
-            if (row < a.R) {
-                const long long d = (long long)s_part[0][ct][j][lane] + s_part[1][ct][j][lane] + s_part[2][ct][j][lane] +
-                                    s_part[3][ct][j][lane];
-                const unsigned long long kv = ((unsigned long long)(na_m + nb_r[jj] - 2 * d) << 16) | var_r[jj];
-                best = kv < best ? kv : best;
-            }
+            const uint32_t kv = ((uint32_t)(na_m + nb_r[jj] - 2 * dot[jj]) << 5) | var_r[jj];
+            if (row < a.R && m < N) best = min(best, kv);
         }
     }
-    {
-        const unsigned long long o = __shfl_xor(best, 32, 64);
-        best = o < best ? o : best;
-    }
+    best = min(best, (uint32_t)__shfl_xor((int)best, 32, 64));
     if (lane < 32) s_key[wave][lane] = best;
     __syncthreads();
     // neuron c's key: the minimum of the two waves that hold its column tile; best match: first minimum of
     // the distances (Trainer.h:164-168), found by every wave for itself
-    auto key_of = [&](uint32_t c) {
-        const unsigned long long k0 = s_key[c >> 5][c & 31], k1 = s_key[(c >> 5) + 2][c & 31];
-        return k1 < k0 ? k1 : k0;
-    };
-    unsigned long long cand = ~0ull;
-    if (lane < N) cand = ((key_of(lane) >> 16) << 8) | lane;
-    const uint32_t bmu = (uint32_t)(wave_min_u64(cand) & 255u);
-    const uint32_t r = (uint32_t)(key_of(n) & 0xffffu);
+    auto key_of = [&](uint32_t c) { return min(s_key[c >> 5][c & 31], s_key[(c >> 5) + 2][c & 31]); };
+    uint32_t dist = lane < N ? key_of(lane) >> 5 : 0xffffffffu, lowest = dist;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) lowest = min(lowest, (uint32_t)__shfl_xor((int)lowest, o, 64));
+    const uint32_t bmu = (uint32_t)__builtin_ctzll(__ballot(dist == lowest));
+    const uint32_t r = key_of(n) & 31u;
     const float f = s_f[bmu];
     if (n == 0 && tid == 0) {
         *a.bmu_out = bmu;
@@ -1410,31 +1416,25 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
     }
 
     // (4) update (Trainer.h:175) and the neuron's row of the next SOM operand
-    const uint32_t D = max(a.vp.D, 1u);
     const uint32_t flip = r >= a.vp.num_rot ? 1u : 0u, rem = r - flip * a.vp.num_rot;
     const uint32_t q = rem / a.vp.nrr, i = rem - q * a.vp.nrr;
     const float *x = s_var + (size_t)((q & 1) * a.vp.nrr + i) * S;
-    const uint32_t rev_x = flip ^ (q >> 1), rev_y = q >> 1;
-    const RcpDivisor by_DD(D * D), by_D(D);
-    long long sq = 0;
+    const uint32_t shift = 16 * (2 * (flip ^ (q >> 1)) + (q >> 1));       // rows reversed, columns reversed
+    signed char *row_next = Pa_next + ((((size_t)(n >> 5) * KS) * 64 + (n & 31)) << 4);
+    int sq = 0;
 #pragma unroll
     for (int u = 0; u < EPT; ++u) {
         const uint32_t j = tid + 256 * u;
         if (j < S) {
             float nv = wv[u];
             if (f != 0.0f) {
-                uint32_t c, p, qx, qy;
-                by_DD.divmod(j, c, p);
-                by_D.divmod(p, qx, qy);
-                const uint32_t src = j - p + (rev_x ? D - 1 - qx : qx) * D + (rev_y ? D - 1 - qy : qy);
+                const uint32_t src = (uint32_t)(sp[u] >> shift) & 0xffffu;
                 nv = __fsub_rn(nv, __fmul_rn(__fsub_rn(nv, x[src]), f));
                 som[(size_t)n * S + j] = nv;
             }
-            const uint32_t k = kk[u];
-            if (k != 0xffffffffu) {
+            if (kb[u] != 0xffffffffu) {
                 const int h = quantise(nv, 255.0f) - 128;
-                const size_t byte = ((((size_t)(n >> 5) * KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
-                Pa_next[byte] = (signed char)h;
+                row_next[kb[u]] = (signed char)h;
                 sq += h * h;
             }
         }
@@ -1443,7 +1443,7 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
     for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
     if (lane == 0) s_sq[wave] = sq;
     __syncthreads();
-    if (tid == 0) a.na_next[n] = s_sq[0] + s_sq[1] + s_sq[2] + s_sq[3];
+    if (tid == 0) a.na_next[n] = (long long)s_sq[0] + s_sq[1] + s_sq[2] + s_sq[3];
 }
 
 // Decode keys: distance (optionally square-rooted for the mapper, Mapper.h:206), exact
@@ -1554,6 +1554,8 @@ struct pink_hip_ctx {
     v4i *d_gPa_alt = nullptr;             // small uint8 trainers: the SOM operand alternates between two buffers
     uint32_t pa_cur = 0;                   // ... which of them holds the current SOM
     bool small_train = false;              // ... one launch per image (k_train_small_u8)
+    unsigned long long *d_src4 = nullptr;  // ... its per-element tables (see the kernel)
+    uint32_t *d_kbyte = nullptr;
     uint32_t *d_grow = nullptr, *d_gvariant = nullptr;   // variant index -> row of the variant operand, and back
     long long *d_gna = nullptr, *d_gnb = nullptr;
     int *d_dot = nullptr;
@@ -2027,7 +2029,7 @@ int run_train_small(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     const size_t lds = (size_t)a.nstored * ctx->S * sizeof(float);
 #define LAUNCH_SMALL(...)                                                                                        \
     hipLaunchKernelGGL((k_train_small_u8<__VA_ARGS__>), dim3(ctx->N), dim3(256), lds, ctx->stream, ctx->d_som, rot, pa, pa_next, pb, \
-                       ctx->d_factors, ctx->d_inv, a)
+                       ctx->d_factors, ctx->d_src4, ctx->d_kbyte, a)
     // (elements per thread, k-steps a wave holds at a time: one batch of operand loads up to 32 k-steps)
     if (ctx->S <= 1024) LAUNCH_SMALL(4, 8); else LAUNCH_SMALL(8, 8);
 #undef LAUNCH_SMALL
@@ -2055,7 +2057,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
@@ -2509,6 +2511,27 @@ int init_ctx(pink_hip_ctx *ctx)
             const size_t a_vec = (size_t)(ctx->Np / 32) * ctx->gKS * 64;
             TRY(dev_alloc(ctx, &ctx->d_gPa_alt, a_vec));
             HIP_TRY(ctx, hipMemset(ctx->d_gPa_alt, 0, a_vec * sizeof(v4i)));
+            std::vector<unsigned long long> src4(ctx->S);
+            std::vector<uint32_t> kbyte(ctx->S);
+            const uint32_t D = ctx->D;
+            for (uint32_t j = 0; j < ctx->S; ++j) {
+                const uint32_t p = j % (D * D), qx = p / D, qy = p % D;
+                unsigned long long packed = 0;
+                for (uint32_t combo = 0; combo < 4; ++combo) {
+                    const uint32_t src = j - p + ((combo >> 1) ? D - 1 - qx : qx) * D + ((combo & 1) ? D - 1 - qy : qy);
+                    packed |= (unsigned long long)src << (16 * combo);
+                }
+                src4[j] = packed;
+                const uint32_t k = inv[j];
+                kbyte[j] = k == 0xffffffffu ? k : (k >> 5) * 1024 + ((k >> 4) & 1) * 512 + (k & 15);
+            }
+            TRY(dev_alloc(ctx, &ctx->d_src4, src4.size()));
+            TRY(dev_alloc(ctx, &ctx->d_kbyte, kbyte.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_src4, src4.data(), src4.size() * sizeof(unsigned long long), hipMemcpyHostToDevice));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_kbyte, kbyte.data(), kbyte.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+            // (limits are per kernel, not per context)
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
         }
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
