@@ -242,7 +242,8 @@ class Context:
 
     def train(self, images, want_bmu=True):
         """Train on the images in order.  want_bmu=False returns nothing and, for up to 128 KiB of
-        images, does not wait for the GPU (see update_counts / synchronize / get_som)."""
+        images, only copies them: they are trained in order a launch group at a time, when the group is full or
+        another call on the context follows (update_counts / synchronize / get_som wait for the result)."""
         images = np.ascontiguousarray(images, np.float32)
         n = images.size // self.image_size
         assert n * self.image_size == images.size

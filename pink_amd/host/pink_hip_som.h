@@ -185,7 +185,8 @@ public:
         uint32_t channels = 0, image_dim = 0;
         hip_detail::image_geometry(data.get_layout(), channels, image_dim);
         auto* ctx = m_device.for_image(channels, image_dim);
-        // nothing is handed back: the library copies the image and returns with the work queued
+        // nothing is handed back: the library copies the image and returns; images are trained in order, a
+        // launch group at a time (when the group is full, or when update_som / get_update_info follows)
         hip_detail::check(ctx, pink_hip_train(ctx, data.get_data_pointer(), 1, nullptr));
     }
 

@@ -265,7 +265,8 @@ class Trainer:
 
     def __call__(self, data):
         """One image (Trainer.h:263-304).  Returns nothing, like the reference, and does not wait for
-        the GPU: the image is copied and the work queued; update_som() and get_update_info() wait."""
+        the GPU: the image is copied, and images are trained in order a launch group at a time (when the group
+        is full, or when update_som() or get_update_info() follows); those two wait for the result."""
         images = self._dev.for_images(np.asarray(data)[None], getattr(data, "layout", "cartesian-2d"))
         self._dev.ctx.train(images, want_bmu=False)
 
