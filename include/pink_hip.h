@@ -161,7 +161,8 @@ int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_i
  * from a static device array of PINK_HIP_STATIC_SCRATCH_BYTES that every GPU holds from the moment the
  * library is loaded until the process ends, not from the context's own allocations; the call itself
  * allocates and frees nothing and clears the part of the array it uses with a kernel.  Images are
- * processed in groups of as many as fit the array; PINK_HIP_EINVAL when a single image of the context
+ * processed in groups of as many as fit the array (less its last KiB, which kernels that read ahead of
+ * their operand may touch); PINK_HIP_EINVAL when a single image of the context
  * does not fit (the message says how many bytes it needs), PINK_HIP_ESTATE on a trainer or while
  * per-kernel timing is on (event records allocate).  All contexts on a GPU share the one array: calls
  * that overlap on the same GPU (two contexts, two streams) race; calls one after the other are fine. */

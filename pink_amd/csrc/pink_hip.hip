@@ -589,153 +589,59 @@ __global__ __launch_bounds__(64) void k_dist_valu(const void *__restrict__ somP_
 
 
 // ---------------------------------------------------------------------------------
-// Float32 distance + argmin: LDS-shared rotations, neuron values broadcast by DPP.
+// Float32 distance + argmin of small problems (about one wave per SIMD): LDS-shared rotations, neuron
+// values broadcast by DPP.
 // A block of 4 waves shares 64 consecutive rotations.  Their packed regions (k contiguous per
 // rotation) are staged through a double-buffered LDS tile of 64 rotations x 64 elements by
-// coalesced 16-byte loads, so every rotation element leaves L2 once per 4*TN neurons; a lane
+// coalesced 16-byte loads, so every rotation element leaves L2 once per 4 neurons; a lane
 // reads its own rotation's row back 16 bytes at a time (row stride 68 words: conflict-free).
-// Wave w owns neurons n0 + w*TN .. + TN, lane l owns rotation r0 + l.  Neuron values travel in
-// VGPRs -- lane l holds element k0 + 16*s + (l % 16) of slab s -- and reach all lanes of a row
-// through the DPP operand of the subtract (`v_sub_f32_dpp ... row_newbcast:k`), so a pair
+// Wave w owns neuron n0 + w, lane l owns rotation r0 + l.  The neuron's 64 values of a chunk come as ONE
+// 16-byte load per lane -- element e in register e % 4 of lane e / 4 of every row of 16 lanes -- and reach
+// all lanes of a row through the DPP operand of the subtract (`v_sub_f32_dpp ... row_newbcast:k`), so a pair
 // element costs exactly one subtract and one fma and no scalar or LDS traffic for the neuron side.
 // The sum of each (neuron, rotation) pair is still one lane's sequential fma chain over k in
 // the CPU's element order (bit-faithful); only the argmin crosses lanes.
+//
+// A lone wave issues one instruction of any kind about every eight clocks, so what is not one of the 128
+// subtracts and multiply-adds of a chunk costs as much as they do: the chunk loop is on an instruction diet
+// (four register sets for the neuron that take turns without copies, addresses that are a uniform base
+// advanced once per four chunks plus per-thread offsets that never change plus a constant, one wait per 16
+// elements) and written as one assembly statement, generated by gen_ssd_steps.py, which says why.  The loads
+// that run ahead are neither branched around nor clamped at the end of a row: they read up to kDistOverrun
+// floats past it, which both operands are allocated with.
 // ---------------------------------------------------------------------------------
 constexpr uint32_t kDistKC = 64;
 constexpr uint32_t kDistRow = kDistKC + 4;   // LDS row stride in floats
 
-// The inner blocks (inline assembly: DPP subtracts issued ahead of the multiply-adds that use
-// them) are generated by gen_ssd_steps.py.
 #include "ssd_steps.inc"
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// HB = rotation values fetched from LDS per batch (64: a whole stage at once, for small TN where a
-// wave has little else to overlap the LDS latency with; 16 otherwise).
-template <int TN, int PD, int HB>
-__global__ __launch_bounds__(256, 4) void k_dist_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
+constexpr uint32_t kDistOverrun = 4 * kDistKC;       // floats that the loads running ahead may read past a row's end
+__global__ __launch_bounds__(256, 2) void k_dist_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                          unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
                                                          uint32_t R, uint32_t Rpad)
 {
     __shared__ v4f s_rot[2][64 * kDistRow / 4];          // [stage][64 rotations][64 elements + 4]
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t r0 = blockIdx.x * kWave;
-    const uint32_t n0 = blockIdx.y * (4 * TN) + wave * TN;
+    const uint32_t n = blockIdx.y * 4 + wave;
     const uint32_t b = blockIdx.z;
-    const float *rp = rotT + ((size_t)b * Rpad + r0) * Epad;
-    const float *np[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) np[j] = somP + (size_t)min(n0 + j, N - 1) * Epad + (lane & 15);
-    float acc[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[j] = 0.0f;
-
-    // Thread t moves 4 vectors of a stage: rotation t/16 + 16*i (i < 4), elements 4*(t & 15) .. +4.
-    // Chunks c+1 .. c+PD are in flight in registers while chunk c is computed from LDS.
+    // thread t stages 4 vectors of a chunk: rotation t / 16 + 16 i (i < 4), elements 4 (t % 16) .. + 4
     const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
-    const float *lp = rp + (size_t)lrow * Epad + lcol;
-    const size_t rstep = (size_t)16 * Epad;
-    const uint32_t lds_w = (lrow * kDistRow + lcol) / 4;      // vector index of this thread's first store
-    const uint32_t lds_wstep = 16 * kDistRow / 4;
-    const uint32_t nchunks = Epad / kDistKC;
-    v4f st[PD][4];
-    float vn[PD][4][TN];     // [slot][slab][neuron]: lane l holds element 16*slab + l%16 of the chunk
-    float va[4][TN];
-
-    {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s_rot[0][lds_w + i * lds_wstep] = *(const v4f *)(lp + i * rstep);
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl) va[sl][j] = np[j][16 * sl];
-#pragma unroll
-        for (int u = 0; u < PD; ++u) {
-            if (u + 1 < nchunks) {
-                const uint32_t k = (u + 1) * kDistKC;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) st[u][i] = *(const v4f *)(lp + k + i * rstep);
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int sl = 0; sl < 4; ++sl) vn[u][sl][j] = np[j][k + 16 * sl];
-            }
-        }
-    }
-    __syncthreads();
-
-#define PINK_SLAB(SL)                                                                                      \
-    {                                                                                                      \
-        if (HB == 16 || (SL) == 0) {                                                                       \
-            /* fetch the next HB elements of this lane's rotation from LDS in one batch, then compute */  \
-            _Pragma("unroll") for (int q = 0; q < HB / 4; ++q) {                                           \
-                const v4f t4 = cur[(SL) * 4 + q];                                                          \
-                bv[4 * q] = t4.x; bv[4 * q + 1] = t4.y; bv[4 * q + 2] = t4.z; bv[4 * q + 3] = t4.w;        \
-            }                                                                                              \
-            __builtin_amdgcn_sched_barrier(0);                                                             \
-        }                                                                                                  \
-        const float *bs = bv + ((SL) * 16) % HB;                                                           \
-        if constexpr (TN == 1) {                                                                           \
-            ssd_block<0>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs);                                  \
-        } else if constexpr (TN == 2) {                                                                    \
-            ssd_block<0>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs);                                  \
-            ssd_block<8>(acc, va[SL], bs); ssd_block<12>(acc, va[SL], bs);                                 \
-        } else if constexpr (TN == 4) {                                                                    \
-            ssd_block<0>(acc, va[SL], bs); ssd_block<2>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs);   \
-            ssd_block<6>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs); ssd_block<10>(acc, va[SL], bs);  \
-            ssd_block<12>(acc, va[SL], bs); ssd_block<14>(acc, va[SL], bs);                                \
-        } else {                                                                                           \
-            ssd_block<0>(acc, va[SL], bs); ssd_block<1>(acc, va[SL], bs); ssd_block<2>(acc, va[SL], bs);   \
-            ssd_block<3>(acc, va[SL], bs); ssd_block<4>(acc, va[SL], bs); ssd_block<5>(acc, va[SL], bs);   \
-            ssd_block<6>(acc, va[SL], bs); ssd_block<7>(acc, va[SL], bs); ssd_block<8>(acc, va[SL], bs);   \
-            ssd_block<9>(acc, va[SL], bs); ssd_block<10>(acc, va[SL], bs); ssd_block<11>(acc, va[SL], bs); \
-            ssd_block<12>(acc, va[SL], bs); ssd_block<13>(acc, va[SL], bs); ssd_block<14>(acc, va[SL], bs);\
-            ssd_block<15>(acc, va[SL], bs);                                                                \
-        }                                                                                                  \
-    }
-
-    for (uint32_t c0 = 0; c0 < nchunks; c0 += PD) {
-#pragma unroll
-        for (int u = 0; u < PD; ++u) {
-            const uint32_t c = c0 + u;          // chunk c+1 waits in register slot u
-            if (c < nchunks) {
-                const v4f *cur = s_rot[c & 1] + lane * (kDistRow / 4);
-                float bv[HB];
-                // (a VALU write of a DPP source needs two idle slots before the DPP read: every
-                // generated block begins with the no-op that provides them)
-                PINK_SLAB(0) PINK_SLAB(1) PINK_SLAB(2) PINK_SLAB(3)
-                if (c + 1 < nchunks) {
-                    v4f *nx = s_rot[(c + 1) & 1];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) nx[lds_w + i * lds_wstep] = st[u][i];
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int sl = 0; sl < 4; ++sl) va[sl][j] = vn[u][sl][j];
-                }
-                if (c + 1 + PD < nchunks) {
-                    const uint32_t k = (c + 1 + PD) * kDistKC;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) st[u][i] = *(const v4f *)(lp + k + i * rstep);
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int sl = 0; sl < 4; ++sl) vn[u][sl][j] = np[j][k + 16 * sl];
-                }
-                __syncthreads();
-            }
-        }
-    }
-#undef PINK_SLAB
+    const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) v4f *)&s_rot[0][0];
+    float acc = 0.0f;
+    ssd_lone_wave_loop(acc, (lrow * Epad + lcol) * 4, ((lrow + 16) * Epad + lcol) * 4, ((lrow + 32) * Epad + lcol) * 4,
+                       ((lrow + 48) * Epad + lcol) * 4, (lane & 15) * 16, lds + (lrow * kDistRow + lcol) * 4,
+                       lds + lane * kDistRow * 4, rotT + ((size_t)b * Rpad + r0) * Epad, somP + (size_t)min(n, N - 1) * Epad,
+                       Epad / kDistKC);
 
     const uint32_t r = r0 + lane;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        unsigned long long kv = ((unsigned long long)__float_as_uint(acc[j]) << 32) | r;
-        if (r >= R) kv = ~0ull;
-        kv = wave_min_u64(kv);
-        if (lane == 0 && n0 + j < N) atomicMin(&key[(size_t)b * N + n0 + j], kv);
-    }
+    unsigned long long kv = ((unsigned long long)__float_as_uint(acc) << 32) | r;
+    if (r >= R) kv = ~0ull;
+    kv = wave_min_u64(kv);
+    if (lane == 0 && n < N) atomicMin(&key[(size_t)b * N + n], kv);
 }
 
 // The same distance for large problems (many waves per SIMD): the neuron values are scalar operands.
@@ -1874,8 +1780,7 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const float *rotT = (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad;
     unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
     if (!scalar_operands) {
-        // (1 neuron per wave, 2 chunks of prefetch, whole-stage LDS batches)
-        hipLaunchKernelGGL((k_dist_f32_dpp<1, 2, 64>), dim3(rblocks, groups(ctx->N, 1), B), dim3(256), 0, ctx->stream,
+        hipLaunchKernelGGL(k_dist_f32_dpp, dim3(rblocks, groups(ctx->N, 1), B), dim3(256), 0, ctx->stream,
                            (const float *)ctx->d_somP, rotT, key, ctx->N, ctx->Epad, ctx->R, ctx->Rpad);
         return;
     }
@@ -2436,8 +2341,9 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, &ctx->d_Pb, B * ctx->RT * ctx->KS * 1024));
         TRY(dev_alloc(ctx, &ctx->d_nb, B * ctx->RT * 32));
     } else {
-        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad));
-        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad));
+        // (the float distance kernel of small problems reads up to kDistOverrun floats past a row's end)
+        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP, (size_t)ctx->N * ctx->Epad + kDistOverrun));
+        TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_rotT, B * ctx->Epad * ctx->Rpad + kDistOverrun));
         // rows beyond R and elements beyond the region must read as zero whoever fills the rest
         HIP_TRY(ctx, hipMemset(ctx->d_rotT, 0, B * ctx->Epad * ctx->Rpad * sizeof(uint32_t)));
         if (ctx->f32gemm) {
@@ -2969,13 +2875,15 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
     if (!ctx->static_scratch) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: no static scratch on this device");
     const StaticPieces pc = static_pieces(ctx);
     const size_t per_image = pc.per_image();
-    if (per_image > PINK_HIP_STATIC_SCRATCH_BYTES)
+    // (the float distance kernel of small problems reads up to kDistOverrun floats past the last row of its
+    // operand, the piece carved last)
+    const size_t capacity = PINK_HIP_STATIC_SCRATCH_BYTES - kDistOverrun * sizeof(float);
+    if (per_image > capacity)
         return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device_static: one image of this context needs " + std::to_string(per_image) +
-                                          " bytes of scratch, the static scratch holds " +
-                                          std::to_string((size_t)PINK_HIP_STATIC_SCRATCH_BYTES));
+                                          " bytes of scratch, the static scratch holds " + std::to_string(capacity));
     if (n_images == 0) return PINK_HIP_OK;
     HIP_TRY(ctx, hipSetDevice(ctx->device));
-    const uint32_t B = (uint32_t)std::min<size_t>({(size_t)ctx->Bcap, PINK_HIP_STATIC_SCRATCH_BYTES / per_image, (size_t)n_images});
+    const uint32_t B = (uint32_t)std::min<size_t>({(size_t)ctx->Bcap, capacity / per_image, (size_t)n_images});
 
     // the scratch keeps what the last call (of any context on this GPU) left: rows beyond the last variant
     // and elements beyond the region must read as zero, so the part this call uses starts from zero
