@@ -9,12 +9,16 @@ BV = 32            # v[32:95]   the lane's 64 rotation values of the chunk being
 DT = 96            # v[96:103]  eight differences in flight
 ST = (104, 120)    # v[104:119], v[120:135]  rotation vectors of the chunks c + 1 and c + 2 on their way to LDS
 NV = 136           # v[136:151] the neuron's chunks c .. c + 3, four registers each
-S_RP, S_NP, S_CNT = 40, 42, 44      # s[40:41] rotation rows, s[42:43] neuron row, s44 chunks left
+XV = 152           # v[152:167] (updating form) the same chunks of the variant that the neuron is pulled toward
+S_RP, S_NP, S_CNT, S_F, S_XP, S_WP = 40, 42, 44, 45, 46, 48   # s[40:41] rotation rows, s[42:43] neuron row, s44 chunks left,
+                                                              # s45 update factor, s[46:47] variant row, s[48:49] new neuron row
 STAGE = 64 * 68 * 4                 # bytes of one LDS stage: 64 rows of 64 + 4 floats
 ROWS16 = 16 * 68 * 4                # bytes between a thread's four staging vectors (16 rows)
+PLAIN, UPDATE, COPY = 0, 1, 2
+NAMES = {PLAIN: "ssd_lone_wave_loop", UPDATE: "ssd_lone_wave_loop_update", COPY: "ssd_lone_wave_loop_copy"}
 
 
-def lone_wave_loop():
+def lone_wave_loop(mode):
     """The whole chunk loop of the kernel for small problems (one neuron per wave, about one wave per SIMD) as
     ONE asm statement.  A lone wave issues an instruction of any kind about every eight clocks, so the loop is
     written down to the instruction: per 64-element chunk 64 DPP subtracts, 64 multiply-adds, 16 LDS reads,
@@ -25,88 +29,151 @@ def lone_wave_loop():
 
     Element e of a chunk of the neuron sits in register e % 4 of lane e / 4 of every row of 16 lanes (one
     16-byte load per lane) and reaches all lanes of the row as the DPP operand of the subtract; every
-    (neuron, rotation) sum is one lane's multiply-add chain in element order.  No DPP source is written by
-    the vector ALU (the loads write them), so no idle slots are needed before the subtracts.
+    (neuron, rotation) sum is one lane's multiply-add chain in element order.
 
-    Loads issued per chunk c: four rotation vectors of chunk c + 3, then the neuron vector of chunk c + 4
-    (the prologue issues the same sequence).  Behind the neuron vector of chunk c come 15 loads before chunk
-    c needs it (11 in the prologue behind that of chunk 0; the first four of the 15 are rotation vectors that
-    chunk c - 1 has already waited for, so the one wait for "at most 11 outstanding" serves both), behind the
-    rotation vectors of chunk c + 1 come 6 before chunk c stores them to LDS.  The last chunk issues nothing;
-    the loads of the three chunks before it read past the end of the rows."""
-    A = []
+    Three forms.  PLAIN computes the distances.  UPDATE first pulls the neuron toward a variant x with factor
+    f -- w = w - ((w - x) * f), three roundings, per chunk one more load (x, fetched alongside the neuron) and
+    twelve vector-ALU instructions ahead of the subtracts (the last write of a neuron register is more than the
+    two idle slots a DPP read needs before its first use) -- stores the new chunk of the neuron's row to a
+    second buffer and computes the distances to the new values.  COPY stores the chunk unchanged.  All lanes
+    store: the four rows of 16 lanes write the same bytes to the same place.
+
+    Memory operations issued per chunk c, in this order: the store of chunk c (UPDATE, COPY), four rotation
+    vectors of chunk c + 3, the neuron vector of chunk c + 4, the variant vector of chunk c + 4 (UPDATE); the
+    prologue issues the loads of the chunks before in the same order.  Vector memory operations complete in the
+    order of issue, so "at most n outstanding" waits for everything but the last n: the n of every wait is
+    counted below over the prologue and three passes of the loop, the smallest count of a place is the one
+    that holds in all of them (a smaller n waits for older operations too, which by then have long arrived).
+    The last chunk issues no loads; the loads of the three chunks before it read past the end of the rows."""
+    upd, store = mode == UPDATE, mode != PLAIN
     def vr(base, n=4):
         return "v[%d:%d]" % (base, base + n - 1)
-    def gload(dst, voff, sbase, imm):
-        A.append("global_load_dwordx4 %s, %s, s[%d:%d]%s" % (vr(dst), voff, sbase, sbase + 1, " offset:%d" % imm if imm else ""))
-    A.append("s_mov_b64 s[%d:%d], %%[rp]" % (S_RP, S_RP + 1))
-    A.append("s_mov_b64 s[%d:%d], %%[np]" % (S_NP, S_NP + 1))
-    A.append("s_mov_b32 s%d, %%[cnt]" % S_CNT)
+    def gload(dst, voff, sbase, imm, tag):
+        return {"text": "global_load_dwordx4 %s, %s, s[%d:%d]%s" % (vr(dst), voff, sbase, sbase + 1, " offset:%d" % imm if imm else ""),
+                "vm": tag}
+    def plain(text):
+        return {"text": text}
+    def wait(tags, lgkm=None):
+        return {"wait": tags, "lgkm": lgkm}
+
+    pro = [plain("s_mov_b64 s[%d:%d], %%[rp]" % (S_RP, S_RP + 1)), plain("s_mov_b64 s[%d:%d], %%[np]" % (S_NP, S_NP + 1)),
+           plain("s_mov_b32 s%d, %%[cnt]" % S_CNT)]
+    if upd:
+        pro += [plain("s_mov_b64 s[%d:%d], %%[xp]" % (S_XP, S_XP + 1)), plain("s_mov_b32 s%d, %%[f]" % S_F)]
+    if store:
+        pro.append(plain("s_mov_b64 s[%d:%d], %%[wp]" % (S_WP, S_WP + 1)))
+    def neuron_loads(u, imm, c):
+        out = [gload(NV + 4 * u, "%[noff]", S_NP, imm, ("nv", c))]
+        if upd:
+            out.append(gload(XV + 4 * u, "%[noff]", S_XP, imm, ("xv", c)))
+        return out
     for i in range(4):
-        gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0)              # chunk 0 of the rotations, through the chunk registers
-    gload(NV + 0, "%[noff]", S_NP, 0)
-    gload(NV + 4, "%[noff]", S_NP, 256)
+        pro.append(gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0, ("st", 0)))       # chunk 0 of the rotations, through the chunk registers
+    pro += neuron_loads(0, 0, 0) + neuron_loads(1, 256, 1)
+    pro += [gload(ST[0] + 4 * i, "%%[roff%d]" % i, S_RP, 256, ("st", 1)) for i in range(4)]
+    pro += neuron_loads(2, 512, 2)
+    pro += [gload(ST[1] + 4 * i, "%%[roff%d]" % i, S_RP, 512, ("st", 2)) for i in range(4)]
+    pro += neuron_loads(3, 768, 3)
+    pro.append(wait([("st", 0)]))
     for i in range(4):
-        gload(ST[0] + 4 * i, "%%[roff%d]" % i, S_RP, 256)
-    gload(NV + 8, "%[noff]", S_NP, 512)
-    for i in range(4):
-        gload(ST[1] + 4 * i, "%%[roff%d]" % i, S_RP, 512)
-    gload(NV + 12, "%[noff]", S_NP, 768)
-    A.append("s_waitcnt vmcnt(12)")
-    for i in range(4):
-        A.append("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else ""))
-    A.append("s_waitcnt lgkmcnt(0)")
-    A.append("s_barrier")
-    A.append("0:")
-    for u in range(4):
+        pro.append(plain("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else "")))
+    pro += [plain("s_waitcnt lgkmcnt(0)"), plain("s_barrier"), plain("0:")]
+
+    def chunk(u, c):        # chunk c = 4 * pass + u; tags are absolute so that the counting below can find them
+        out = []
         rd, wr = (u & 1) * STAGE, ((u + 1) & 1) * STAGE
         for q in range(16):
             off = rd + 16 * q
-            A.append("ds_read_b128 %s, %%[ldsr]%s" % (vr(BV + 4 * q), " offset:%d" % off if off else ""))
-        nv = NV + 4 * u
+            out.append(plain("ds_read_b128 %s, %%[ldsr]%s" % (vr(BV + 4 * q), " offset:%d" % off if off else "")))
+        nv, xv = NV + 4 * u, XV + 4 * u
+        mine = [("nv", c)] + ([("xv", c)] if upd else [])
+        if store:
+            out.append(wait(mine))
+            if upd:
+                out += [plain("v_sub_f32_e32 v%d, v%d, v%d" % (DT + r, nv + r, xv + r)) for r in range(4)]
+                out += [plain("v_mul_f32_e32 v%d, s%d, v%d" % (DT + r, S_F, DT + r)) for r in range(4)]
+                out += [plain("v_sub_f32_e32 v%d, v%d, v%d" % (nv + r, nv + r, DT + r)) for r in range(4)]
+            out.append({"text": "global_store_dwordx4 %%[noff], %s, s[%d:%d]%s" % (vr(nv), S_WP, S_WP + 1, " offset:%d" % (u * 256) if u else ""),
+                        "vm": ("wr", c)})
         for sl in range(4):
             # (the neuron vector with the first slab; the rotation vectors that go to LDS behind the last slab with it)
-            A.append("s_waitcnt %slgkmcnt(%d)" % ("vmcnt(11) " if sl == 0 else "vmcnt(6) " if sl == 3 else "", 12 - 4 * sl))
+            out.append(wait(mine if sl == 0 and not store else [("st", c + 1)] if sl == 3 else [], 12 - 4 * sl))
             def sub(e):
-                return "v_sub_f32_dpp v%d, v%d, v%d row_newbcast:%d row_mask:0xf bank_mask:0xf" % (
-                    DT + (e & 7), nv + (e & 3), BV + 16 * sl + e, 4 * sl + e // 4)
+                return plain("v_sub_f32_dpp v%d, v%d, v%d row_newbcast:%d row_mask:0xf bank_mask:0xf" % (
+                    DT + (e & 7), nv + (e & 3), BV + 16 * sl + e, 4 * sl + e // 4))
             def fma(e):
-                return "v_fmac_f32_e32 %%[acc], v%d, v%d" % (DT + (e & 7), DT + (e & 7))
-            A.extend(sub(e) for e in range(8))
+                return plain("v_fmac_f32_e32 %%[acc], v%d, v%d" % (DT + (e & 7), DT + (e & 7)))
+            out += [sub(e) for e in range(8)]
             for e in range(8):
-                A.extend([fma(e), sub(8 + e)])
-            A.extend(fma(8 + e) for e in range(8))
-        A.append("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1))
-        A.append("s_cbranch_scc1 1f")
+                out += [fma(e), sub(8 + e)]
+            out += [fma(8 + e) for e in range(8)]
+        out += [plain("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1)), plain("s_cbranch_scc1 1f")]
         st = ST[u & 1]
-        for i in range(4):
-            A.append("ds_write_b128 %%[ldsw], %s offset:%d" % (vr(st + 4 * i), wr + i * ROWS16))
-        for i in range(4):
-            gload(st + 4 * i, "%%[roff%d]" % i, S_RP, (u + 3) * 256)
-        gload(nv, "%[noff]", S_NP, (u + 4) * 256)
-        A.append("s_waitcnt lgkmcnt(0)")
-        A.append("s_barrier")
+        out += [plain("ds_write_b128 %%[ldsw], %s offset:%d" % (vr(st + 4 * i), wr + i * ROWS16)) for i in range(4)]
+        out += [gload(st + 4 * i, "%%[roff%d]" % i, S_RP, (u + 3) * 256, ("st", c + 3)) for i in range(4)]
+        out += neuron_loads(u, (u + 4) * 256, c + 4)
+        out += [plain("s_waitcnt lgkmcnt(0)"), plain("s_barrier")]
+        return out
+
+    # the n of every wait: operations issued behind the last one it waits for, the fewest over the passes
+    passes = 3
+    stream = list(pro)
+    sites = {}                               # (u, index in the chunk) -> counts seen
+    for ps in range(passes):
+        for u in range(4):
+            for k, item in enumerate(chunk(u, 4 * ps + u)):
+                item = dict(item)
+                item["site"] = (u, k)
+                stream.append(item)
+    counts = {}
+    for pos, item in enumerate(stream):
+        if "wait" not in item or not item["wait"]:
+            continue
+        last = max(i for i in range(pos) if stream[i].get("vm") in item["wait"])
+        assert all(any(stream[i].get("vm") == t for i in range(pos)) for t in item["wait"])
+        behind = sum(1 for i in range(last + 1, pos) if "vm" in stream[i])
+        key = item.get("site", ("pro", pos))
+        counts[key] = min(counts.get(key, 1 << 30), behind)
+    def wait_text(item, key):
+        parts = []
+        if item["wait"]:
+            parts.append("vmcnt(%d)" % counts[key])
+        if item.get("lgkm") is not None:
+            parts.append("lgkmcnt(%d)" % item["lgkm"])
+        return "s_waitcnt " + " ".join(parts)
+    A = []
+    for pos, item in enumerate(pro):
+        A.append(wait_text(item, ("pro", pos)) if "wait" in item else item["text"])
+    for u in range(4):
+        for k, item in enumerate(chunk(u, u)):
+            A.append(wait_text(item, (u, k)) if "wait" in item else item["text"])
     A.append("s_sub_u32 s%d, s%d, 4" % (S_CNT, S_CNT))
-    for sb in (S_RP, S_NP):
+    for sb in [S_RP, S_NP] + ([S_XP] if upd else []) + ([S_WP] if store else []):
         A.append("s_add_u32 s%d, s%d, 0x400" % (sb, sb))
         A.append("s_addc_u32 s%d, s%d, 0" % (sb + 1, sb + 1))
     A.append("s_branch 0b")
     A.append("1:")
     A.append("s_waitcnt vmcnt(0)")
+
+    name = NAMES[mode]
+    extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f", COPY: ", float *wp"}[mode]
+    extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f)', COPY: ', [wp] "s"(wp)'}[mode]
     lines = []
-    lines.append("// The chunk loop of the kernel for small problems, one neuron per wave (see gen_ssd_steps.py).")
-    lines.append("// roff: byte offsets of the thread's four staging vectors in a chunk of the block's 64 rotation rows; noff: byte")
-    lines.append("// offset of the lane's neuron vector in a chunk; ldsw, ldsr: LDS byte addresses of the thread's first staging")
-    lines.append("// vector and of the lane's row in stage 0; rp, np: chunk 0 of the rotation rows and of the neuron row; chunks >= 1.")
-    lines.append("__device__ __forceinline__ void ssd_lone_wave_loop(float &acc, uint32_t roff0, uint32_t roff1, uint32_t roff2, uint32_t roff3,")
-    lines.append("                                                   uint32_t noff, uint32_t ldsw, uint32_t ldsr, const float *rp, const float *np,")
-    lines.append("                                                   uint32_t chunks)")
+    lines.append({PLAIN: "// The chunk loop of the kernel for small problems, one neuron per wave (see gen_ssd_steps.py).",
+                  UPDATE: "// The same loop, the neuron pulled toward the variant row xp with factor f first and its new row stored to wp.",
+                  COPY: "// The same loop, the neuron's row also stored to wp as it is."}[mode])
+    if mode == PLAIN:
+        lines.append("// roff: byte offsets of the thread's four staging vectors in a chunk of the block's 64 rotation rows; noff: byte")
+        lines.append("// offset of the lane's neuron vector in a chunk; ldsw, ldsr: LDS byte addresses of the thread's first staging")
+        lines.append("// vector and of the lane's row in stage 0; rp, np: chunk 0 of the rotation rows and of the neuron row; chunks >= 1.")
+    lines.append("__device__ __forceinline__ void %s(float &acc, uint32_t roff0, uint32_t roff1, uint32_t roff2, uint32_t roff3," % name)
+    lines.append("        uint32_t noff, uint32_t ldsw, uint32_t ldsr, const float *rp, const float *np, uint32_t chunks%s)" % extra_args)
     lines.append("{")
     lines.append("    asm volatile(" + "\n        ".join('"%s\\n\\t"' % a for a in A))
     lines.append('        : [acc] "+v"(acc)')
     lines.append('        : [roff0] "v"(roff0), [roff1] "v"(roff1), [roff2] "v"(roff2), [roff3] "v"(roff3), [noff] "v"(noff), [ldsw] "v"(ldsw),')
-    lines.append('          [ldsr] "v"(ldsr), [rp] "s"(rp), [np] "s"(np), [cnt] "s"(chunks)')
-    clob = ['"v%d"' % r for r in range(BV, NV + 16)] + ['"s%d"' % r for r in range(S_RP, S_CNT + 1)] + ['"scc"', '"memory"']
+    lines.append('          [ldsr] "v"(ldsr), [rp] "s"(rp), [np] "s"(np), [cnt] "s"(chunks)%s' % extra_ops)
+    clob = ['"v%d"' % r for r in range(BV, (XV if upd else NV) + 16)] + ['"s%d"' % r for r in range(S_RP, S_WP + 2)] + ['"scc"', '"memory"']
     rows = [", ".join(clob[i:i + 16]) for i in range(0, len(clob), 16)]
     lines.append("        : " + ",\n          ".join(rows) + ");")
     lines.append("}")
@@ -114,5 +181,6 @@ def lone_wave_loop():
 
 
 print("// Generated by gen_ssd_steps.py -- do not edit.")
-print()
-print(lone_wave_loop())
+for mode in (PLAIN, UPDATE, COPY):
+    print()
+    print(lone_wave_loop(mode))

@@ -644,6 +644,110 @@ __global__ __launch_bounds__(256, 2) void k_dist_f32_dpp(const float *__restrict
     if (lane == 0 && n < N) atomicMin(&key[(size_t)b * N + n], kv);
 }
 
+// One launch per image for small float32 trainers: the distances of image i against the SOM as image i - 1
+// leaves it.  The update of image i - 1 costs a launch of its own about a third of the distance kernel's time
+// (each of its blocks waits for the keys, searches the best match, then waits for its factor); here every
+// wave applies it to its neuron on the fly instead -- w = w - ((w - x) * f) on each chunk of the neuron's
+// operand row as it arrives, x the same chunk of the row of the variant of image i - 1 that was closest to the
+// neuron -- and stores the new row to the other of two operand buffers (all waves of a neuron store the same
+// bytes; an untouched neuron's row is copied).  What a wave needs for it does not depend on the search: the
+// keys of image i - 1 and the neuron's whole column of the factor matrix are requested together, the best
+// match is the minimum over the wave, the factor comes out of the column by lane.  The neuron's full image
+// (all elements, not only the region that the operand row holds) is not on this path: k_update_replay applies
+// the updates of a group of images to it in one launch, in order.
+struct PrevImage {
+    const unsigned long long *key;      // keys of image i - 1 (null: nothing to apply)
+    const float *rotT;                  // its packed variants
+    const float *factors;
+    float *somP_next;
+    uint32_t *bmu_out, *counts;
+};
+
+__global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
+                                                          unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
+                                                          uint32_t R, uint32_t Rpad, PrevImage prev)
+{
+    __shared__ v4f s_rot[2][64 * kDistRow / 4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t r0 = blockIdx.x * kWave;
+    const uint32_t n = blockIdx.y * 4 + wave, nc = min(n, N - 1);
+    const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
+    const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) v4f *)&s_rot[0][0];
+    const uint32_t roff0 = (lrow * Epad + lcol) * 4, roff1 = ((lrow + 16) * Epad + lcol) * 4,
+                   roff2 = ((lrow + 32) * Epad + lcol) * 4, roff3 = ((lrow + 48) * Epad + lcol) * 4;
+    const uint32_t noff = (lane & 15) * 16, ldsw = lds + (lrow * kDistRow + lcol) * 4, ldsr = lds + lane * kDistRow * 4;
+    const float *rp = rotT + (size_t)r0 * Epad, *np = somP + (size_t)nc * Epad;
+    const uint32_t chunks = Epad / kDistKC;
+    float acc = 0.0f;
+    if (prev.key == nullptr) {
+        ssd_lone_wave_loop(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks);
+    } else {
+        // (N <= 256: four keys and four factors per lane; every load is issued before the first is used, indices
+        // past the end are clamped and dropped afterwards)
+        const uint32_t *key32 = (const uint32_t *)prev.key;          // little endian: rotation, then the distance bits
+        uint32_t dist[4];
+        float fcol[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t m = min(lane + 64 * q, N - 1);
+            dist[q] = key32[2 * m + 1];
+            fcol[q] = prev.factors[(size_t)m * N + nc];
+        }
+        const uint32_t r = key32[2 * nc];                            // the neuron's closest variant of image i - 1
+        // (the loop's first requests, made here as well: they travel while the search below runs, and the loop
+        // finds the lines near)
+        const v4f warm0 = *(const v4f *)((const char *)rp + roff0), warm1 = *(const v4f *)((const char *)rp + roff1),
+                  warm2 = *(const v4f *)((const char *)rp + roff2), warm3 = *(const v4f *)((const char *)rp + roff3),
+                  warm4 = *(const v4f *)((const char *)np + noff);
+        // The best match: the smallest distance of the wave (a reduction over the lanes by DPP: within quads, rows
+        // of 16, then across the rows into lane 63; no LDS round trips), then the first neuron that has it.
+        uint32_t dmin = 0xffffffffu;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (lane + 64 * q >= N) dist[q] = 0xffffffffu;
+            dmin = min(dmin, dist[q]);
+        }
+#define PINK_DPP_MIN(ctrl, rows) \
+    dmin = min(dmin, (uint32_t)__builtin_amdgcn_update_dpp((int)0xffffffffu, (int)dmin, ctrl, rows, 0xf, false))
+        PINK_DPP_MIN(0xb1, 0xf);      // quad_perm [1, 0, 3, 2]
+        PINK_DPP_MIN(0x4e, 0xf);      // quad_perm [2, 3, 0, 1]
+        PINK_DPP_MIN(0x141, 0xf);     // row_half_mirror
+        PINK_DPP_MIN(0x140, 0xf);     // row_mirror
+        PINK_DPP_MIN(0x142, 0xa);     // row_bcast:15 into rows 1 and 3
+        PINK_DPP_MIN(0x143, 0xc);     // row_bcast:31 into rows 2 and 3
+#undef PINK_DPP_MIN
+        const uint32_t best = (uint32_t)__builtin_amdgcn_readlane((int)dmin, 63);
+        uint32_t bmu = 0;
+        float f = 0.0f;
+#pragma unroll
+        for (int q = 3; q >= 0; --q) {
+            const unsigned long long hit = __ballot(dist[q] == best && lane + 64 * q < N);
+            if (hit) {
+                const uint32_t at = (uint32_t)__builtin_ctzll(hit);
+                bmu = at + 64 * q;
+                f = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, fcol[q]), (int)at));
+            }
+        }
+        if (blockIdx.x == 0 && n == 0 && lane == 0) {
+            *prev.bmu_out = bmu;
+            atomicAdd(&prev.counts[bmu], 1u);          // m_update_info[bmu]++ (Trainer.h:302-303)
+        }
+        asm volatile("" ::"v"(warm0), "v"(warm1), "v"(warm2), "v"(warm3), "v"(warm4));
+        float *wp = prev.somP_next + (size_t)nc * Epad;
+        if (f == 0.0f)
+            ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
+        else
+            ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks,
+                                      prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad, wp, f);
+    }
+    const uint32_t rr = r0 + lane;
+    unsigned long long kv = ((unsigned long long)__float_as_uint(acc) << 32) | rr;
+    if (rr >= R) kv = ~0ull;
+    kv = wave_min_u64(kv);
+    if (lane == 0 && n < N) atomicMin(&key[n], kv);
+}
+
 // The same distance for large problems (many waves per SIMD): the neuron values are scalar operands.
 // A DPP operand halves the issue rate of the subtract (measured: 5.9 against 3.2 clocks per instruction
 // with eight waves per SIMD), which a lone wave does not notice -- it issues only every other turn anyway --
@@ -1168,6 +1272,63 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     }
 }
 
+// The neurons' full images after a group of images: thread (n, j) pulls element j of neuron n toward the
+// closest variant of image 0, then of image 1, ... (Trainer.h:164-179; CudaLib/update_neurons.h), with the
+// arithmetic of k_update.  The best match of image i is bmu[i]; the closest variant of the neuron is in its
+// key.  Nothing here waits for a search: one launch replays what k_update does in one launch per image.  What
+// an image contributes to neuron n -- factor, row of the stored variant, how it is read -- is worked out for
+// all images side by side first (one thread each) and kept in LDS, so the loop over the images is one
+// variant element and three operations per image with nothing that depends on the image before.
+constexpr uint32_t kReplayMax = 256;         // images per launch
+__global__ __launch_bounds__(256) void k_update_replay(float *__restrict__ som, const float *__restrict__ rot,
+                                                       const unsigned long long *__restrict__ key, const float *__restrict__ factors,
+                                                       const uint32_t *__restrict__ bmu, uint32_t images, uint32_t N, uint32_t S,
+                                                       uint32_t R, uint32_t shift, VariantPair vp)
+{
+    __shared__ float s_f[kReplayMax];
+    __shared__ uint32_t s_row[kReplayMax];   // stored row of the group's variants * 4 + how it is read
+    const uint32_t n = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
+    if (threadIdx.x < images) {
+        const uint32_t i = threadIdx.x;
+        const uint32_t r = (uint32_t)(key[(size_t)i * N + n] & ((1ull << shift) - 1ull));
+        uint32_t row = r, which = 0;
+        if (vp.D) {
+            // stored: the base rotation and its quarter turn; the others are those with rows and / or columns reversed
+            const uint32_t fl = r >= vp.num_rot ? 1u : 0u, rem = r - fl * vp.num_rot;
+            const uint32_t q = rem / vp.nrr, b = rem - q * vp.nrr;
+            row = (q & 1) * vp.nrr + b;
+            which = 2 * (fl ^ (q >> 1)) + (q >> 1);
+        }
+        s_f[i] = factors[(size_t)bmu[i] * N + n];
+        s_row[i] = (i * R + row) * 4 + which;
+    }
+    __syncthreads();
+    if (j >= S) return;
+    // where element j sits in a stored variant read as it is, with columns, rows or both reversed (see k_update)
+    uint32_t src[4] = {j, j, j, j};
+    if (vp.D) {
+        const uint32_t D = vp.D, p = j % (D * D), x = p / D, y = p % D;
+        src[1] = j - p + x * D + (D - 1 - y);
+        src[2] = j - p + (D - 1 - x) * D + y;
+        src[3] = j - p + (D - 1 - x) * D + (D - 1 - y);
+    }
+    float w = som[(size_t)n * S + j];
+    for (uint32_t i0 = 0; i0 < images; i0 += 8) {
+        float x[8], f[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t i = min(i0 + u, images - 1);
+            const uint32_t rw = s_row[i], which = rw & 3;
+            f[u] = i0 + u < images ? s_f[i] : 0.0f;
+            x[u] = rot[(size_t)(rw >> 2) * S + (which == 0 ? src[0] : which == 1 ? src[1] : which == 2 ? src[2] : src[3])];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u)
+            if (f[u] != 0.0f) w = __fsub_rn(w, __fmul_rn(__fsub_rn(w, x[u]), f[u]));
+    }
+    som[(size_t)n * S + j] = w;
+}
+
 // ---------------------------------------------------------------------------------
 // Small uint8 trainers (at most 64 neurons and 32 variants, e.g. 8 x 8 neurons of 28 x 28 pixels under
 // the eight symmetries): the whole step of an image -- distances, best match, update, operand refresh --
@@ -1407,6 +1568,11 @@ struct pink_hip_ctx {
     uint32_t *d_region = nullptr;
     unsigned long long *d_key = nullptr;
     void *d_somP = nullptr, *d_rotT = nullptr;
+    // small float32 trainers: one launch per image, the SOM operand alternates between two buffers (d_somP is
+    // always the current one), the best matches of a group of images in d_bmu_group (see k_train_f32_dpp)
+    bool fused_f32_train = false;
+    void *d_somP_alt = nullptr;
+    uint32_t *d_bmu_group = nullptr;
     uint32_t *d_bmu_scratch = nullptr;
     uint32_t *d_inv = nullptr;   // element of a neuron -> position in the region (none: ~0); null if not one-to-one
     float *d_dist = nullptr;
@@ -1914,6 +2080,43 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     return launch_check(ctx, "k_update");
 }
 
+// Distances of the image in slot `slot` against the SOM with the update of the image before it applied on the
+// way (small float32 trainers, k_train_f32_dpp); that image's best match goes to *bmu_prev.
+int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu_prev)
+{
+    Timed t(ctx, kClsDist);
+    PrevImage prev{};
+    if (has_prev) {
+        prev.key = ctx->d_key + (size_t)(slot - 1) * ctx->N;
+        prev.rotT = (const float *)ctx->d_rotT + (size_t)(slot - 1) * ctx->Epad * ctx->Rpad;
+        prev.factors = ctx->d_factors;
+        prev.somP_next = (float *)ctx->d_somP_alt;
+        prev.bmu_out = bmu_prev;
+        prev.counts = ctx->d_counts;
+    }
+    hipLaunchKernelGGL(k_train_f32_dpp, dim3(ctx->Rpad / kWave, (ctx->N + 3) / 4), dim3(256), 0, ctx->stream,
+                       (const float *)ctx->d_somP, (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad,
+                       ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, prev);
+    if (has_prev) std::swap(ctx->d_somP, ctx->d_somP_alt);        // the updated operand is the current one now
+    return launch_check(ctx, "k_train_f32_dpp");
+}
+
+// The updates of the first `images` images of the current group applied to the neurons' full images, in order.
+int run_update_replay(pink_hip_ctx *ctx, uint32_t images, const uint32_t *dev_bmu)
+{
+    Timed t(ctx, kClsUpdate);
+    VariantPair vp{};
+    if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
+    for (uint32_t first = 0; first < images; first += kReplayMax) {
+        const uint32_t count = std::min(kReplayMax, images - first);
+        hipLaunchKernelGGL(k_update_replay, dim3((ctx->S + 255) / 256, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
+                           ctx->d_rot + (size_t)first * ctx->R * ctx->S, ctx->d_key + (size_t)first * ctx->N, ctx->d_factors,
+                           dev_bmu + first, count, ctx->N, ctx->S, ctx->R, ctx->shift, vp);
+        TRY(launch_check(ctx, "k_update_replay"));
+    }
+    return PINK_HIP_OK;
+}
+
 // Distances, best match and update of the image in slot `slot` in one launch (small uint8 trainers).
 int run_train_small(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
 {
@@ -1960,7 +2163,7 @@ int free_all(pink_hip_ctx *ctx)
     for (auto &p : ctx->events) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
-                    ctx->d_somP, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
+                    ctx->d_somP, ctx->d_somP_alt, ctx->d_bmu_group, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
                     ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
@@ -2439,6 +2642,13 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
         }
+        // one launch per image where the float32 distance kernel runs in its one-wave-per-SIMD form (see k_train_f32_dpp)
+        ctx->fused_f32_train = c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv && ctx->N <= 256 &&
+                               (size_t)(ctx->Rpad / kWave) * ((ctx->N + 3) / 4) <= (size_t)4 * ctx->num_cu;
+        if (ctx->fused_f32_train) {
+            TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP_alt, (size_t)ctx->N * ctx->Epad + kDistOverrun));
+            TRY(dev_alloc(ctx, &ctx->d_bmu_group, B));
+        }
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
@@ -2669,6 +2879,15 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
         const uint32_t B = std::min(ctx->Bcap, n_images - done);
         TRY(run_rotate(ctx, dev_images + (size_t)done * ctx->isz, B, ctx->pair_variants ? kStorePair : kStoreAll));
         TRY(run_pack_rot(ctx, B));
+        if (ctx->fused_f32_train) {
+            // every launch but the first applies the update of the image before it; the last image's update and,
+            // ahead of it, all the others on the neurons' full images close the group
+            uint32_t *bmu = dev_bmu_out ? dev_bmu_out + done : ctx->d_bmu_group;
+            for (uint32_t b = 0; b < B; ++b) TRY(run_train_f32(ctx, b, b > 0, b > 0 ? bmu + b - 1 : nullptr));
+            if (B > 1) TRY(run_update_replay(ctx, B - 1, bmu));
+            TRY(run_update(ctx, B - 1, bmu + B - 1));
+            continue;
+        }
         for (uint32_t b = 0; b < B; ++b) {
             if (ctx->small_train) {
                 TRY(run_train_small(ctx, b, dev_bmu_out ? dev_bmu_out + done + b : ctx->d_bmu_scratch));
