@@ -456,6 +456,12 @@ FUSED_TRAIN_SHAPES = [
     (5, 2, 14, 12, 1, True, 9, capi.QUADRATIC, capi.UINT8, 4),        # one rotation and its flip, two channels
     (7, 1, 14, 12, 1, False, 9, capi.QUADRATIC, capi.UINT8, 3),       # a single variant
     (40, 1, 20, 20, 8, True, 20, capi.QUADRATIC, capi.UINT8, 7),      # an odd number of images: the SOM operand ends in its second buffer
+    # small float32 trainers: the distance launch of an image applies the update of the image before it
+    (70, 1, 20, 14, 32, True, 9, capi.CIRCULAR, capi.FLOAT, 5),       # three chunks of 64 elements, neurons not a multiple of four
+    (9, 1, 12, 8, 16, True, 8, capi.QUADRATIC, capi.FLOAT, 4),        # a single chunk
+    (130, 2, 16, 11, 4, True, 11, capi.QUADRATIC, capi.FLOAT, 3),     # two channels, three keys per lane in the search
+    (256, 1, 14, 10, 8, False, 10, capi.QUADRATIC, capi.FLOAT, 3),    # the most neurons that train this way
+    (257, 1, 14, 10, 8, False, 10, capi.QUADRATIC, capi.FLOAT, 3),    # ... and one more
 ]
 
 
