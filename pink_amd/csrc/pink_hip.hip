@@ -2484,6 +2484,15 @@ int init_ctx(pink_hip_ctx *ctx)
         size_t b = c.max_batch ? c.max_batch : 64;
         const size_t budget = (size_t)2 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
+        if (!c.max_batch) {
+            // a group's variants and operands are written by one launch and read back image by image: a group that
+            // stays within the 256 MB last-level cache trains faster (measured: 10 x 10 float32 +2.6 % with 48
+            // against 64 images, the hexagonal uint16 SOM +5 % with 16 against 32; groups below 16 cost the
+            // rotation kernel more than they save)
+            const size_t stored = ctx->pair_variants ? std::min<size_t>(2 * std::max(ctx->nrr, 1u), ctx->R) : ctx->R;
+            const size_t touched = per_image - (ctx->R - stored) * ctx->S * 4;
+            while (b > 16 && b * touched > ((size_t)224 << 20)) b -= std::min<size_t>(8, b - 16);
+        }
         ctx->Bcap = (uint32_t)b;
     } else {
         size_t b = c.max_batch ? c.max_batch : ((ctx->mfma || ctx->mfma_sym) ? 2048 : 256);
