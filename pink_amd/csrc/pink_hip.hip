@@ -1272,6 +1272,79 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     }
 }
 
+// The update of a float32 trainer on the distance operand alone: block (part, n) finds the best match like k_update,
+// then pulls its slice of neuron n's operand row toward the packed row of the neuron's closest variant (the same
+// elements in the same order: no index arithmetic, 16-byte accesses).  The neurons' full images follow once per
+// group of images (k_update_replay): the distance never reads them.
+__global__ __launch_bounds__(256) void k_update_rows(float *__restrict__ somP, const float *__restrict__ rotT,
+                                                     const unsigned long long *__restrict__ key, const float *__restrict__ factors,
+                                                     uint32_t *__restrict__ bmu_out, uint32_t *__restrict__ counts, uint32_t N,
+                                                     uint32_t Epad, uint32_t parts, uint32_t shift)
+{
+    __shared__ unsigned long long s_val[4];
+    __shared__ uint32_t s_idx[4];
+    const uint32_t tid = threadIdx.x, n = blockIdx.y, part = blockIdx.x;
+    unsigned long long bv = ~0ull;
+    uint32_t bi = 0xffffffffu;
+    for (uint32_t m = tid; m < N; m += 256) {
+        const unsigned long long v = key[m] >> shift;
+        if (v < bv) { bv = v; bi = m; }        // ascending index per thread: first minimum kept
+    }
+    const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
+    // the slice's first round of loads does not depend on the search: requested ahead of it
+    const uint32_t vecs = Epad / 4, chunk = (vecs + parts - 1) / parts;
+    const uint32_t v0 = part * chunk, v1 = min(vecs, v0 + chunk);
+    v4f *__restrict__ w = (v4f *)(somP + (size_t)n * Epad);
+    const v4f *__restrict__ x = (const v4f *)(rotT + (size_t)r * Epad);
+    constexpr uint32_t U = 4;
+    v4f wv[U], xv[U];
+    auto load_round = [&](uint32_t vb) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t v = vb + 256 * u;
+            if (v < v1) { wv[u] = w[v]; xv[u] = x[v]; }
+        }
+    };
+    load_round(v0 + tid);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const unsigned long long ov = __shfl_xor(bv, o, 64);
+        const uint32_t oi = __shfl_xor(bi, o, 64);
+        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if ((tid & 63) == 0) { s_val[tid >> 6] = bv; s_idx[tid >> 6] = bi; }
+    __syncthreads();
+    bv = s_val[0]; bi = s_idx[0];
+#pragma unroll
+    for (int g = 1; g < 4; ++g) {
+        const unsigned long long ov = s_val[g];
+        const uint32_t oi = s_idx[g];
+        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const uint32_t bmu = bi;
+    if (n == 0 && part == 0 && tid == 0) {
+        *bmu_out = bmu;
+        atomicAdd(&counts[bmu], 1u);           // m_update_info[bmu]++ (Trainer.h:302-303)
+    }
+    const float f = factors[(size_t)bmu * N + n];
+    if (f == 0.0f) return;
+    for (uint32_t vb = v0 + tid; vb < v1; vb += 256 * U) {
+        if (vb != v0 + tid) load_round(vb);
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            const uint32_t v = vb + 256 * u;
+            if (v < v1) {
+                v4f o;
+                o.x = __fsub_rn(wv[u].x, __fmul_rn(__fsub_rn(wv[u].x, xv[u].x), f));
+                o.y = __fsub_rn(wv[u].y, __fmul_rn(__fsub_rn(wv[u].y, xv[u].y), f));
+                o.z = __fsub_rn(wv[u].z, __fmul_rn(__fsub_rn(wv[u].z, xv[u].z), f));
+                o.w = __fsub_rn(wv[u].w, __fmul_rn(__fsub_rn(wv[u].w, xv[u].w), f));
+                w[v] = o;
+            }
+        }
+    }
+}
+
 // The neurons' full images after a group of images: thread (n, j) pulls element j of neuron n toward the
 // closest variant of image 0, then of image 1, ... (Trainer.h:164-179; CudaLib/update_neurons.h), with the
 // arithmetic of k_update.  The best match of image i is bmu[i]; the closest variant of the neuron is in its
@@ -1573,6 +1646,9 @@ struct pink_hip_ctx {
     bool fused_f32_train = false;
     void *d_somP_alt = nullptr;
     uint32_t *d_bmu_group = nullptr;
+    // the other float32 trainers on the vector ALU: per image the update of the SOM operand alone (k_update_rows), the
+    // neurons' full images once per group
+    bool rows_f32_train = false;
     uint32_t *d_bmu_scratch = nullptr;
     uint32_t *d_inv = nullptr;   // element of a neuron -> position in the region (none: ~0); null if not one-to-one
     float *d_dist = nullptr;
@@ -2099,6 +2175,20 @@ int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu
                        ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, prev);
     if (has_prev) std::swap(ctx->d_somP, ctx->d_somP_alt);        // the updated operand is the current one now
     return launch_check(ctx, "k_train_f32_dpp");
+}
+
+// The update of the image in slot `slot` on the float32 distance operand alone (k_update_rows).
+int run_update_rows(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
+{
+    Timed t(ctx, kClsUpdate);
+    const uint32_t vecs = ctx->Epad / 4;
+    const uint32_t target_blocks = (size_t)ctx->N * ctx->Epad >= ((size_t)1 << 20) ? 1024u : 128u;
+    uint32_t parts = (target_blocks + ctx->N - 1) / ctx->N;
+    parts = std::max(1u, std::min(parts, (vecs + 255) / 256));
+    hipLaunchKernelGGL(k_update_rows, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, (float *)ctx->d_somP,
+                       (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad, ctx->d_key + (size_t)slot * ctx->N,
+                       ctx->d_factors, dev_bmu_out, ctx->d_counts, ctx->N, ctx->Epad, parts, ctx->shift);
+    return launch_check(ctx, "k_update_rows");
 }
 
 // The updates of the first `images` images of the current group applied to the neurons' full images, in order.
@@ -2654,10 +2744,10 @@ int init_ctx(pink_hip_ctx *ctx)
         // one launch per image where the float32 distance kernel runs in its one-wave-per-SIMD form (see k_train_f32_dpp)
         ctx->fused_f32_train = c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv && ctx->N <= 256 &&
                                (size_t)(ctx->Rpad / kWave) * ((ctx->N + 3) / 4) <= (size_t)4 * ctx->num_cu;
-        if (ctx->fused_f32_train) {
-            TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP_alt, (size_t)ctx->N * ctx->Epad + kDistOverrun));
-            TRY(dev_alloc(ctx, &ctx->d_bmu_group, B));
-        }
+        ctx->rows_f32_train = !ctx->fused_f32_train && c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv &&
+                              B <= kReplayMax;
+        if (ctx->fused_f32_train) TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP_alt, (size_t)ctx->N * ctx->Epad + kDistOverrun));
+        if (ctx->fused_f32_train || ctx->rows_f32_train) TRY(dev_alloc(ctx, &ctx->d_bmu_group, B));
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
@@ -2895,6 +2985,15 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
             for (uint32_t b = 0; b < B; ++b) TRY(run_train_f32(ctx, b, b > 0, b > 0 ? bmu + b - 1 : nullptr));
             if (B > 1) TRY(run_update_replay(ctx, B - 1, bmu));
             TRY(run_update(ctx, B - 1, bmu + B - 1));
+            continue;
+        }
+        if (ctx->rows_f32_train) {
+            uint32_t *bmu = dev_bmu_out ? dev_bmu_out + done : ctx->d_bmu_group;
+            for (uint32_t b = 0; b < B; ++b) {
+                TRY(run_dist(ctx, b, 1));
+                TRY(run_update_rows(ctx, b, bmu + b));
+            }
+            TRY(run_update_replay(ctx, B, bmu));
             continue;
         }
         for (uint32_t b = 0; b < B; ++b) {
