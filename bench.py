@@ -51,10 +51,11 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg0", "update"): ((27.486e6 + 0.774e6 + 1.590e6 + 1.184e6) / 64, "profiles/cfg0_train_f32_counters.txt"),   # per group of 64
     ("cfg1", "rotate"): ((95.060e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg1", "distance"): ((214.633e6 + 1.639e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg2", "distance"): (26.949e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (25.158e6 + 20.721e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (640.430e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg3", "update"): (104.827e6 + 140.439e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg2", "distance"): (26.958e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (25.150e6 + 20.722e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg3", "distance"): (876.388e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
+    ("cfg3", "update"): (63.762e6 + 47.153e6 + (998.532e6 + 95.565e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
     ("cfg4", "update"): (1.210e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
 }
 
