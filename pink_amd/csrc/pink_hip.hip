@@ -68,6 +68,31 @@ __device__ __forceinline__ unsigned long long wave_min_u64(unsigned long long v)
     return v;
 }
 
+// Minimum of a 32-bit value over the wave by DPP (within quads, rows of 16, then across the rows into lane 63):
+// no LDS round trips, for waves that have their SIMD to themselves and pay for every instruction's latency.
+__device__ __forceinline__ uint32_t wave_min_u32_dpp(uint32_t v)
+{
+#define PINK_DPP_MIN(ctrl, rows) \
+    v = min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)0xffffffffu, (int)v, ctrl, rows, 0xf, false))
+    PINK_DPP_MIN(0xb1, 0xf);      // quad_perm [1, 0, 3, 2]
+    PINK_DPP_MIN(0x4e, 0xf);      // quad_perm [2, 3, 0, 1]
+    PINK_DPP_MIN(0x141, 0xf);     // row_half_mirror
+    PINK_DPP_MIN(0x140, 0xf);     // row_mirror
+    PINK_DPP_MIN(0x142, 0xa);     // row_bcast:15 into rows 1 and 3
+    PINK_DPP_MIN(0x143, 0xc);     // row_bcast:31 into rows 2 and 3
+#undef PINK_DPP_MIN
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// The key `bits << 32 | first + lane` of the lane with the smallest bits (the first such lane), lanes with
+// valid == false left out; all ones when no lane is valid.
+__device__ __forceinline__ unsigned long long wave_min_key_dpp(uint32_t bits, bool valid, uint32_t first)
+{
+    const uint32_t best = wave_min_u32_dpp(valid ? bits : 0xffffffffu);
+    const unsigned long long hit = __ballot(valid && bits == best);
+    return hit ? ((unsigned long long)best << 32) | (first + (uint32_t)__builtin_ctzll(hit)) : ~0ull;
+}
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
@@ -637,10 +662,8 @@ __global__ __launch_bounds__(256, 2) void k_dist_f32_dpp(const float *__restrict
                        lds + lane * kDistRow * 4, rotT + ((size_t)b * Rpad + r0) * Epad, somP + (size_t)min(n, N - 1) * Epad,
                        Epad / kDistKC);
 
-    const uint32_t r = r0 + lane;
-    unsigned long long kv = ((unsigned long long)__float_as_uint(acc) << 32) | r;
-    if (r >= R) kv = ~0ull;
-    kv = wave_min_u64(kv);
+    // (float bits of a sum of squares order like the floats; rotations past the last one are left out)
+    const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
     if (lane == 0 && n < N) atomicMin(&key[(size_t)b * N + n], kv);
 }
 
@@ -700,24 +723,15 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         const v4f warm0 = *(const v4f *)((const char *)rp + roff0), warm1 = *(const v4f *)((const char *)rp + roff1),
                   warm2 = *(const v4f *)((const char *)rp + roff2), warm3 = *(const v4f *)((const char *)rp + roff3),
                   warm4 = *(const v4f *)((const char *)np + noff);
-        // The best match: the smallest distance of the wave (a reduction over the lanes by DPP: within quads, rows
-        // of 16, then across the rows into lane 63; no LDS round trips), then the first neuron that has it.
+        // The best match: the smallest distance of the wave (a reduction over the lanes by DPP), then the first
+        // neuron that has it.
         uint32_t dmin = 0xffffffffu;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             if (lane + 64 * q >= N) dist[q] = 0xffffffffu;
             dmin = min(dmin, dist[q]);
         }
-#define PINK_DPP_MIN(ctrl, rows) \
-    dmin = min(dmin, (uint32_t)__builtin_amdgcn_update_dpp((int)0xffffffffu, (int)dmin, ctrl, rows, 0xf, false))
-        PINK_DPP_MIN(0xb1, 0xf);      // quad_perm [1, 0, 3, 2]
-        PINK_DPP_MIN(0x4e, 0xf);      // quad_perm [2, 3, 0, 1]
-        PINK_DPP_MIN(0x141, 0xf);     // row_half_mirror
-        PINK_DPP_MIN(0x140, 0xf);     // row_mirror
-        PINK_DPP_MIN(0x142, 0xa);     // row_bcast:15 into rows 1 and 3
-        PINK_DPP_MIN(0x143, 0xc);     // row_bcast:31 into rows 2 and 3
-#undef PINK_DPP_MIN
-        const uint32_t best = (uint32_t)__builtin_amdgcn_readlane((int)dmin, 63);
+        const uint32_t best = wave_min_u32_dpp(dmin);
         uint32_t bmu = 0;
         float f = 0.0f;
 #pragma unroll
@@ -741,10 +755,7 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
             ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks,
                                       prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad, wp, f);
     }
-    const uint32_t rr = r0 + lane;
-    unsigned long long kv = ((unsigned long long)__float_as_uint(acc) << 32) | rr;
-    if (rr >= R) kv = ~0ull;
-    kv = wave_min_u64(kv);
+    const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
     if (lane == 0 && n < N) atomicMin(&key[n], kv);
 }
 
