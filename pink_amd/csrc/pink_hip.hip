@@ -84,6 +84,31 @@ __device__ __forceinline__ uint32_t wave_min_u32_dpp(uint32_t v)
     return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
+// The smallest 64-bit value of the wave and the smallest index among the lanes that hold it, the same way: the
+// high words, then the low words of the lanes that are still in, then their indices.
+__device__ __forceinline__ void wave_first_min_u64_dpp(unsigned long long &v, uint32_t &idx)
+{
+    const uint32_t hi = (uint32_t)(v >> 32), lo = (uint32_t)v;
+    const uint32_t mh = wave_min_u32_dpp(hi);
+    const uint32_t ml = wave_min_u32_dpp(hi == mh ? lo : 0xffffffffu);
+    idx = wave_min_u32_dpp(hi == mh && lo == ml ? idx : 0xffffffffu);
+    v = ((unsigned long long)mh << 32) | ml;
+}
+
+// Sum of a 32-bit integer over the wave, the same way.
+__device__ __forceinline__ int wave_sum_i32_dpp(int v)
+{
+#define PINK_DPP_ADD(ctrl, rows) v += __builtin_amdgcn_update_dpp(0, v, ctrl, rows, 0xf, false)
+    PINK_DPP_ADD(0xb1, 0xf);      // pairs
+    PINK_DPP_ADD(0x4e, 0xf);      // quads
+    PINK_DPP_ADD(0x141, 0xf);     // halves of a row
+    PINK_DPP_ADD(0x140, 0xf);     // rows
+    PINK_DPP_ADD(0x142, 0xa);     // row 0 into 1, row 2 into 3
+    PINK_DPP_ADD(0x143, 0xc);     // rows 0 + 1 into 2 and 3
+#undef PINK_DPP_ADD
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // The key `bits << 32 | first + lane` of the lane with the smallest bits (the first such lane), lanes with
 // valid == false left out; all ones when no lane is valid.
 __device__ __forceinline__ unsigned long long wave_min_key_dpp(uint32_t bits, bool valid, uint32_t first)
@@ -1203,13 +1228,8 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         }
     };
     load_round(j0 + tid);
-    // first minimum of the block: within a wave by shuffles, then across the four waves
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-        const unsigned long long ov = __shfl_xor(bv, o, 64);
-        const uint32_t oi = __shfl_xor(bi, o, 64);
-        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    // first minimum of the block: within a wave by DPP, then across the four waves
+    wave_first_min_u64_dpp(bv, bi);
     if ((tid & 63) == 0) { s_val[tid >> 6] = bv; s_idx[tid >> 6] = bi; }
     __syncthreads();
     bv = s_val[0]; bi = s_idx[0];
@@ -1317,12 +1337,7 @@ __global__ __launch_bounds__(256) void k_update_rows(float *__restrict__ somP, c
         }
     };
     load_round(v0 + tid);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-        const unsigned long long ov = __shfl_xor(bv, o, 64);
-        const uint32_t oi = __shfl_xor(bi, o, 64);
-        if (ov < bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    wave_first_min_u64_dpp(bv, bi);
     if ((tid & 63) == 0) { s_val[tid >> 6] = bv; s_idx[tid >> 6] = bi; }
     __syncthreads();
     bv = s_val[0]; bi = s_idx[0];
@@ -1555,9 +1570,7 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
     // neuron c's key: the minimum of the two waves that hold its column tile; best match: first minimum of
     // the distances (Trainer.h:164-168), found by every wave for itself
     auto key_of = [&](uint32_t c) { return min(s_key[c >> 5][c & 31], s_key[(c >> 5) + 2][c & 31]); };
-    uint32_t dist = lane < N ? key_of(lane) >> 5 : 0xffffffffu, lowest = dist;
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) lowest = min(lowest, (uint32_t)__shfl_xor((int)lowest, o, 64));
+    const uint32_t dist = lane < N ? key_of(lane) >> 5 : 0xffffffffu, lowest = wave_min_u32_dpp(dist);
     const uint32_t bmu = (uint32_t)__builtin_ctzll(__ballot(dist == lowest));
     const uint32_t r = key_of(n) & 31u;
     const float f = s_f[bmu];
@@ -1590,8 +1603,7 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
             }
         }
     }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    sq = wave_sum_i32_dpp(sq);
     if (lane == 0) s_sq[wave] = sq;
     __syncthreads();
     if (tid == 0) a.na_next[n] = (long long)s_sq[0] + s_sq[1] + s_sq[2] + s_sq[3];
