@@ -706,7 +706,7 @@ __global__ __launch_bounds__(256, 2) void k_dist_f32_dpp(const float *__restrict
 struct PrevImage {
     const unsigned long long *key;      // keys of image i - 1 (null: nothing to apply)
     const float *rotT;                  // its packed variants
-    const float *factors;
+    const float *factors_t;             // the factor matrix transposed: a neuron's column is contiguous
     float *somP_next;
     uint32_t *bmu_out, *counts;
 };
@@ -740,7 +740,7 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         for (int q = 0; q < 4; ++q) {
             const uint32_t m = min(lane + 64 * q, N - 1);
             dist[q] = key32[2 * m + 1];
-            fcol[q] = prev.factors[(size_t)m * N + nc];
+            fcol[q] = prev.factors_t[(size_t)nc * N + m];
         }
         const uint32_t r = key32[2 * nc];                            // the neuron's closest variant of image i - 1
         // (the loop's first requests, made here as well: they travel while the search below runs, and the loop
@@ -1148,10 +1148,12 @@ struct UpdatePlanes {
     uint32_t KS, Np, u16;
 };
 
+constexpr uint32_t kFactorColumnMax = 2048;      // neurons whose column of the factor matrix a block keeps in LDS
+
 template <uint32_t U>     // elements per thread and round: all their loads are issued before the first store
 __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const float *__restrict__ rot,
                                                 const unsigned long long *__restrict__ key,
-                                                const float *__restrict__ factors, uint32_t *__restrict__ bmu_out,
+                                                const float *__restrict__ factors_t, uint32_t *__restrict__ bmu_out,
                                                 uint32_t N, uint32_t S, uint32_t parts, uint32_t shift,
                                                 void *__restrict__ somP, const uint32_t *__restrict__ inv,
                                                 uint32_t Epad, float qfactor, UpdatePlanes up,
@@ -1159,8 +1161,13 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
 {
     __shared__ unsigned long long s_val[256];
     __shared__ uint32_t s_idx[256];
+    __shared__ float s_fcol[kFactorColumnMax];
     const uint32_t tid = threadIdx.x;
     const uint32_t n = blockIdx.y, part = blockIdx.x;
+    // The factor of this neuron depends on the best match, the neuron's column of the factor matrix does not: it is
+    // requested with the keys (factors_t is the matrix transposed, so the column is contiguous) and waits in LDS.
+    const float *__restrict__ fcol = factors_t + (size_t)n * N;
+    const bool column_in_lds = N <= kFactorColumnMax;
     // What the block will read does not depend on the best-matching neuron, only whether it is
     // needed does: the first round of loads is issued ahead of the search, which then runs while
     // they are in flight (a neuron with factor 0 drops them).
@@ -1169,6 +1176,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     uint32_t bi = 0xffffffffu;
     for (uint32_t m = tid; m < N; m += 256) {
         const unsigned long long v = key[m] >> shift;
+        if (column_in_lds) s_fcol[m] = fcol[m];
         if (v < bv) { bv = v; bi = m; }        // ascending index per thread: first minimum kept
     }
     const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
@@ -1245,7 +1253,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         atomicAdd(&counts[bmu], 1u);           // m_update_info[bmu]++ (Trainer.h:302-303)
     }
 
-    const float f = factors[(size_t)bmu * N + n];
+    const float f = column_in_lds ? s_fcol[bmu] : fcol[bmu];
     if (f == 0.0f) {
         // untouched neuron: its operand row stands, its norm moves to the next buffer
         if (up.Pa && part == 0 && tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], (unsigned long long)up.na_cur[n]);
@@ -1308,17 +1316,21 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
 // elements in the same order: no index arithmetic, 16-byte accesses).  The neurons' full images follow once per
 // group of images (k_update_replay): the distance never reads them.
 __global__ __launch_bounds__(256) void k_update_rows(float *__restrict__ somP, const float *__restrict__ rotT,
-                                                     const unsigned long long *__restrict__ key, const float *__restrict__ factors,
+                                                     const unsigned long long *__restrict__ key, const float *__restrict__ factors_t,
                                                      uint32_t *__restrict__ bmu_out, uint32_t *__restrict__ counts, uint32_t N,
                                                      uint32_t Epad, uint32_t parts, uint32_t shift)
 {
     __shared__ unsigned long long s_val[4];
     __shared__ uint32_t s_idx[4];
+    __shared__ float s_fcol[kFactorColumnMax];
     const uint32_t tid = threadIdx.x, n = blockIdx.y, part = blockIdx.x;
+    const float *__restrict__ fcol = factors_t + (size_t)n * N;      // the neuron's column of the factor matrix (see k_update)
+    const bool column_in_lds = N <= kFactorColumnMax;
     unsigned long long bv = ~0ull;
     uint32_t bi = 0xffffffffu;
     for (uint32_t m = tid; m < N; m += 256) {
         const unsigned long long v = key[m] >> shift;
+        if (column_in_lds) s_fcol[m] = fcol[m];
         if (v < bv) { bv = v; bi = m; }        // ascending index per thread: first minimum kept
     }
     const uint32_t r = (uint32_t)(key[n] & ((1ull << shift) - 1ull));
@@ -1352,7 +1364,7 @@ __global__ __launch_bounds__(256) void k_update_rows(float *__restrict__ somP, c
         *bmu_out = bmu;
         atomicAdd(&counts[bmu], 1u);           // m_update_info[bmu]++ (Trainer.h:302-303)
     }
-    const float f = factors[(size_t)bmu * N + n];
+    const float f = column_in_lds ? s_fcol[bmu] : fcol[bmu];
     if (f == 0.0f) return;
     for (uint32_t vb = v0 + tid; vb < v1; vb += 256 * U) {
         if (vb != v0 + tid) load_round(vb);
@@ -1660,7 +1672,7 @@ struct pink_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
 
-    float *d_som = nullptr, *d_rot = nullptr, *d_cos = nullptr, *d_sin = nullptr, *d_factors = nullptr;
+    float *d_som = nullptr, *d_rot = nullptr, *d_cos = nullptr, *d_sin = nullptr, *d_factors = nullptr, *d_factors_t = nullptr;
     uint32_t *d_region = nullptr;
     unsigned long long *d_key = nullptr;
     void *d_somP = nullptr, *d_rotT = nullptr;
@@ -2167,7 +2179,7 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
 #define LAUNCH_UPDATE(U_)                                                                                        \
     hipLaunchKernelGGL(k_update<U_>, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,                   \
-                       ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors, \
+                       ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors_t, \
                        dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,                                \
                        (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,                           \
                        is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp)
@@ -2188,7 +2200,7 @@ int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu
     if (has_prev) {
         prev.key = ctx->d_key + (size_t)(slot - 1) * ctx->N;
         prev.rotT = (const float *)ctx->d_rotT + (size_t)(slot - 1) * ctx->Epad * ctx->Rpad;
-        prev.factors = ctx->d_factors;
+        prev.factors_t = ctx->d_factors_t;
         prev.somP_next = (float *)ctx->d_somP_alt;
         prev.bmu_out = bmu_prev;
         prev.counts = ctx->d_counts;
@@ -2210,7 +2222,7 @@ int run_update_rows(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     parts = std::max(1u, std::min(parts, (vecs + 255) / 256));
     hipLaunchKernelGGL(k_update_rows, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, (float *)ctx->d_somP,
                        (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad, ctx->d_key + (size_t)slot * ctx->N,
-                       ctx->d_factors, dev_bmu_out, ctx->d_counts, ctx->N, ctx->Epad, parts, ctx->shift);
+                       ctx->d_factors_t, dev_bmu_out, ctx->d_counts, ctx->N, ctx->Epad, parts, ctx->shift);
     return launch_check(ctx, "k_update_rows");
 }
 
@@ -2275,7 +2287,7 @@ int free_all(pink_hip_ctx *ctx)
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &p : ctx->events) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
-    void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_region, ctx->d_key,
+    void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_factors_t, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_somP_alt, ctx->d_bmu_group, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
                     ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
@@ -2774,6 +2786,14 @@ int init_ctx(pink_hip_ctx *ctx)
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
+        {
+            // the same matrix transposed: what a neuron receives for every possible best match, contiguous
+            std::vector<float> t((size_t)ctx->N * ctx->N);
+            for (uint32_t m = 0; m < ctx->N; ++m)
+                for (uint32_t k = 0; k < ctx->N; ++k) t[(size_t)k * ctx->N + m] = c.update_factors[(size_t)m * ctx->N + k];
+            TRY(dev_alloc(ctx, &ctx->d_factors_t, t.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_factors_t, t.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
+        }
     }
     HIP_TRY(ctx, hipDeviceSynchronize());   // set-up copies ran on the null stream
     TRY(run_pack_som(ctx));
