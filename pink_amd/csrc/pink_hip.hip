@@ -1209,6 +1209,9 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         by_DD.divmod(j0 + tid, c, p);
         by_D.divmod(p, px, py);
     }
+    // element (px, py) of a channel plane is read at (rev_x ? D-1-px : px, rev_y ? D-1-py : py): j + c0 + cx px + cy py
+    const int cx = rev_x ? -2 * (int)D : 0, cy = rev_y ? -2 : 0;
+    const int c0 = (rev_x ? (int)((D - 1) * D) : 0) + (rev_y ? (int)D - 1 : 0);
     float wv[U], xv[U];
     uint32_t kk[U];
     auto load_round = [&](uint32_t jb) {
@@ -1217,11 +1220,12 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
             const uint32_t j = jb + 256 * u;
             uint32_t src = j;
             if (stepping) {
-                src = j - (px * D + py) + (rev_x ? D - 1 - px : px) * D + (rev_y ? D - 1 - py : py);
+                src = (uint32_t)((int)j + c0 + __mul24(cx, (int)px) + __mul24(cy, (int)py));
                 py += step_y;
                 px += step_x + (py >= D ? 1u : 0u);
                 py -= py >= D ? D : 0u;
-                while (px >= D) px -= D;           // (past the end of a channel plane: the next one; twice for D < 16)
+                px -= px >= D ? D : 0u;            // (past the end of a channel plane: the next one)
+                if (D < 32) while (px >= D) px -= D;       // (a step of 256 elements spans more than two rows)
             } else if (reversed) {
                 uint32_t c, p, qx, qy;
                 by_DD.divmod(j, c, p);
@@ -1261,24 +1265,25 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     }
     long long sq = 0;
     const size_t plane_bytes = (size_t)(up.Np / 32) * up.KS * 64 * 16;
+    signed char *row_planes = up.Pa + ((((size_t)(n >> 5) * up.KS) * 64 + (n & 31)) << 4);
     // keep the distance kernel's packed copy of the region current (inv = position of element j in
-    // the region, or none)
+    // the region, for the byte planes its byte inside the neuron's row of fragments, or none)
     auto refresh = [&](uint32_t k, float nv) {
         if (k == 0xffffffffu) return;
         if (up.Pa) {
+            // (k: the element's byte inside the neuron's row of fragments; values of at most 17 bits: 24-bit products)
             const int q = quantise(nv, qfactor);
-            const size_t byte = ((((size_t)(n >> 5) * up.KS + (k >> 5)) * 64 + (n & 31) + 32 * ((k & 31) >> 4)) << 4) + (k & 15);
+            signed char *at = row_planes + k;
             if (up.u16) {
                 const int c = q - 32768;
                 const int h = c >> 8, l = (c & 255) - 128;
-                up.Pa[byte] = (signed char)h;
-                up.Pa[plane_bytes + byte] = (signed char)l;
-                const long long v = 256 * h + l;
-                sq += v * v;
+                at[0] = (signed char)h;
+                at[plane_bytes] = (signed char)l;
+                sq += __mul24(c - 128, c - 128);            // (256 h + l) squared
             } else {
                 const int h = q - 128;
-                up.Pa[byte] = (signed char)h;
-                sq += h * h;
+                at[0] = (signed char)h;
+                sq += __mul24(h, h);
             }
         } else if (qfactor > 0.0f) {
             ((int32_t *)somP)[(size_t)n * Epad + k] = quantise(nv, qfactor);
@@ -2181,7 +2186,7 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     hipLaunchKernelGGL(k_update<U_>, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,                   \
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors_t, \
                        dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,                                \
-                       (ctx->gemm && !ctx->fused_som) ? nullptr : ctx->d_inv, ctx->Epad,                           \
+                       ctx->fused_som ? ctx->d_kbyte : ctx->gemm ? nullptr : ctx->d_inv, ctx->Epad,                \
                        is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp)
     // a slice of several rounds keeps eight elements per thread in flight (cfg2 -6 %, cfg3 -3 % against four);
     // a slice of one round is faster with four (cfg0 +8 % with eight)
@@ -2745,6 +2750,17 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipMemcpy(ctx->d_inv, inv.data(), inv.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             ctx->fused_som = ctx->gemm;
         }
+        if (ctx->fused_som) {
+            // where an element of a neuron lands inside the neuron's row of 32-row fragments of the SOM operand
+            // (see k_train_small_u8), or all ones outside the region
+            std::vector<uint32_t> kbyte(ctx->S);
+            for (uint32_t j = 0; j < ctx->S; ++j) {
+                const uint32_t k = inv[j];
+                kbyte[j] = k == 0xffffffffu ? k : (k >> 5) * 1024 + ((k >> 4) & 1) * 512 + (k & 15);
+            }
+            TRY(dev_alloc(ctx, &ctx->d_kbyte, kbyte.size()));
+            HIP_TRY(ctx, hipMemcpy(ctx->d_kbyte, kbyte.data(), kbyte.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        }
         // one launch per image where the whole distance matrix is a few dozen MFMAs (see k_train_small_u8)
         const uint32_t nstored = std::min(2 * std::max(ctx->nrr, 1u), ctx->R);
         ctx->small_train = ctx->fused_som && ctx->pair_variants && c.kernel_choice == PINK_HIP_KERNEL_AUTO &&
@@ -2755,7 +2771,6 @@ int init_ctx(pink_hip_ctx *ctx)
             TRY(dev_alloc(ctx, &ctx->d_gPa_alt, a_vec));
             HIP_TRY(ctx, hipMemset(ctx->d_gPa_alt, 0, a_vec * sizeof(v4i)));
             std::vector<unsigned long long> src4(ctx->S);
-            std::vector<uint32_t> kbyte(ctx->S);
             const uint32_t D = ctx->D;
             for (uint32_t j = 0; j < ctx->S; ++j) {
                 const uint32_t p = j % (D * D), qx = p / D, qy = p % D;
@@ -2765,13 +2780,9 @@ int init_ctx(pink_hip_ctx *ctx)
                     packed |= (unsigned long long)src << (16 * combo);
                 }
                 src4[j] = packed;
-                const uint32_t k = inv[j];
-                kbyte[j] = k == 0xffffffffu ? k : (k >> 5) * 1024 + ((k >> 4) & 1) * 512 + (k & 15);
             }
             TRY(dev_alloc(ctx, &ctx->d_src4, src4.size()));
-            TRY(dev_alloc(ctx, &ctx->d_kbyte, kbyte.size()));
             HIP_TRY(ctx, hipMemcpy(ctx->d_src4, src4.data(), src4.size() * sizeof(unsigned long long), hipMemcpyHostToDevice));
-            HIP_TRY(ctx, hipMemcpy(ctx->d_kbyte, kbyte.data(), kbyte.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             // (limits are per kernel, not per context)
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
