@@ -189,7 +189,9 @@ uint32_t pink_hip_region_size(const pink_hip_ctx *ctx);
 uint32_t pink_hip_distance_kernel(const pink_hip_ctx *ctx);
 
 /* Per-kernel timing with HIP events on the context's stream.  While enabled every
- * launch of the rotation, distance and update kernels is bracketed by two events;
+ * launch of the rotation, distance and update kernels is bracketed by two events
+ * (launches of one kernel that follow each other directly, as a small float32
+ * trainer's one launch per image does within a group, share one pair);
  * pink_hip_kernel_times synchronises and returns, per kernel class, the number of
  * launches and their summed duration in milliseconds since the last reset.
  * Index: 0 rotation, 1 operand packing, 2 distance, 3 update, 4 finalise. */

@@ -1654,7 +1654,7 @@ __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__re
 // ---------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------
-struct EventPair { hipEvent_t a, b; int cls; };
+struct EventPair { hipEvent_t a, b; int cls; uint32_t launches; };
 constexpr size_t kRotateLdsMax = 158 * 1024;
 enum : uint32_t { kStoreNone = 0, kStoreAll = 1, kStorePair = 2 };
 
@@ -1786,8 +1786,9 @@ int fail(pink_hip_ctx *ctx, int code, const std::string &msg)
 struct Timed {
     pink_hip_ctx *ctx;
     int cls;
+    uint32_t launches;      // launches of one kernel queued back to back between the two events
     hipEvent_t a = nullptr, b = nullptr;
-    Timed(pink_hip_ctx *c, int k) : ctx(c), cls(k)
+    Timed(pink_hip_ctx *c, int k, uint32_t n = 1) : ctx(c), cls(k), launches(n)
     {
         if (!ctx->profiling) return;
         auto take = [&]() {
@@ -1804,7 +1805,7 @@ struct Timed {
     {
         if (!ctx->profiling || !a || !b) return;
         (void)hipEventRecord(b, ctx->stream);
-        ctx->events.push_back({a, b, cls});
+        ctx->events.push_back({a, b, cls, launches});
     }
 };
 
@@ -1816,7 +1817,7 @@ int drain_events(pink_hip_ctx *ctx)
         float ms = 0.0f;
         if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
             ctx->prof_ms[p.cls] += ms;
-            ctx->prof_launches[p.cls] += 1;
+            ctx->prof_launches[p.cls] += p.launches;
         }
         ctx->event_pool.push_back(p.a);
         ctx->event_pool.push_back(p.b);
@@ -2200,7 +2201,6 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
 // way (small float32 trainers, k_train_f32_dpp); that image's best match goes to *bmu_prev.
 int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu_prev)
 {
-    Timed t(ctx, kClsDist);
     PrevImage prev{};
     if (has_prev) {
         prev.key = ctx->d_key + (size_t)(slot - 1) * ctx->N;
@@ -3036,7 +3036,11 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
             // every launch but the first applies the update of the image before it; the last image's update and,
             // ahead of it, all the others on the neurons' full images close the group
             uint32_t *bmu = dev_bmu_out ? dev_bmu_out + done : ctx->d_bmu_group;
-            for (uint32_t b = 0; b < B; ++b) TRY(run_train_f32(ctx, b, b > 0, b > 0 ? bmu + b - 1 : nullptr));
+            {
+                // (per-kernel timing: one pair of events around the group's launches, which follow each other directly)
+                Timed t(ctx, kClsDist, B);
+                for (uint32_t b = 0; b < B; ++b) TRY(run_train_f32(ctx, b, b > 0, b > 0 ? bmu + b - 1 : nullptr));
+            }
             if (B > 1) TRY(run_update_replay(ctx, B - 1, bmu));
             TRY(run_update(ctx, B - 1, bmu + B - 1));
             continue;
