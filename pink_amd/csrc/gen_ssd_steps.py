@@ -9,7 +9,8 @@ BV = 32            # v[32:95]   the lane's 64 rotation values of the chunk being
 DT = 96            # v[96:103]  eight differences in flight
 ST = (104, 120)    # v[104:119], v[120:135]  rotation vectors of the chunks c + 1 and c + 2 on their way to LDS
 NV = 136           # v[136:151] the neuron's chunks c .. c + 3, four registers each
-XV = 152           # v[152:167] (updating form) the same chunks of the variant that the neuron is pulled toward
+WL = 152           # v[152:155] (updating form) the neuron's chunks c + 1 .. c + 4, one element per lane
+XL = 156           # v[156:159] (updating form) the same elements of the variant that the neuron is pulled toward
 S_RP, S_NP, S_CNT, S_F, S_XP, S_WP = 40, 42, 44, 45, 46, 48   # s[40:41] rotation rows, s[42:43] neuron row, s44 chunks left,
                                                               # s45 update factor, s[46:47] variant row, s[48:49] new neuron row
 STAGE = 64 * 68 * 4                 # bytes of one LDS stage: 64 rows of 64 + 4 floats
@@ -32,15 +33,17 @@ def lone_wave_loop(mode):
     (neuron, rotation) sum is one lane's multiply-add chain in element order.
 
     Three forms.  PLAIN computes the distances.  UPDATE first pulls the neuron toward a variant x with factor
-    f -- w = w - ((w - x) * f), three roundings, per chunk one more load (x, fetched alongside the neuron) and
-    twelve vector-ALU instructions ahead of the subtracts (the last write of a neuron register is more than the
-    two idle slots a DPP read needs before its first use) -- stores the new chunk of the neuron's row to a
-    second buffer and computes the distances to the new values.  COPY stores the chunk unchanged.  All lanes
-    store: the four rows of 16 lanes write the same bytes to the same place.
+    f -- w = w - ((w - x) * f), three roundings -- stores the new row to a second buffer and computes the distances
+    to the new values.  The update runs one chunk ahead and on one element per lane (lane l holds element l of
+    the chunk: three vector-ALU instructions for the 64 elements, where the layout of the subtract's operand, four
+    elements per lane repeated in every row of 16 lanes, would take twelve): the new chunk goes to memory as it
+    is and through 256 bytes of LDS of the wave's own into the operand layout (one 4-byte write per lane, one
+    16-byte read per lane at the start of the next chunk; LDS operations of a wave complete in order).  COPY
+    stores the chunk unchanged (all lanes store: the four rows of 16 lanes write the same bytes to the same place).
 
-    Memory operations issued per chunk c, in this order: the store of chunk c (UPDATE, COPY), four rotation
-    vectors of chunk c + 3, the neuron vector of chunk c + 4, the variant vector of chunk c + 4 (UPDATE); the
-    prologue issues the loads of the chunks before in the same order.  Vector memory operations complete in the
+    Memory operations issued per chunk c, in this order: the store of chunk c (COPY) or c + 1 (UPDATE), four
+    rotation vectors of chunk c + 3, the neuron's chunk c + 4, the variant's chunk c + 4 (UPDATE); the prologue
+    issues the loads of the chunks before in the same order.  Vector memory operations complete in the
     order of issue, so "at most n outstanding" waits for everything but the last n: the n of every wait is
     counted below over the prologue and three passes of the loop, the smallest count of a place is the one
     that holds in all of them (a smaller n waits for older operations too, which by then have long arrived).
@@ -62,11 +65,19 @@ def lone_wave_loop(mode):
         pro += [plain("s_mov_b64 s[%d:%d], %%[xp]" % (S_XP, S_XP + 1)), plain("s_mov_b32 s%d, %%[f]" % S_F)]
     if store:
         pro.append(plain("s_mov_b64 s[%d:%d], %%[wp]" % (S_WP, S_WP + 1)))
+    def lane_load(dst, sbase, imm, tag):
+        return {"text": "global_load_dword v%d, %%[loff], s[%d:%d]%s" % (dst, sbase, sbase + 1, " offset:%d" % imm if imm else ""), "vm": tag}
     def neuron_loads(u, imm, c):
-        out = [gload(NV + 4 * u, "%[noff]", S_NP, imm, ("nv", c))]
         if upd:
-            out.append(gload(XV + 4 * u, "%[noff]", S_XP, imm, ("xv", c)))
-        return out
+            return [lane_load(WL + u, S_NP, imm, ("wl", c)), lane_load(XL + u, S_XP, imm, ("xl", c))]
+        return [gload(NV + 4 * u, "%[noff]", S_NP, imm, ("nv", c))]
+    def update(u, c, imm):       # chunk c (register set u): the new elements to memory and to the wave's LDS stage c % 2
+        return [wait([("wl", c), ("xl", c)]),
+                plain("v_sub_f32_e32 v%d, v%d, v%d" % (DT, WL + u, XL + u)),
+                plain("v_mul_f32_e32 v%d, s%d, v%d" % (DT, S_F, DT)),
+                plain("v_sub_f32_e32 v%d, v%d, v%d" % (WL + u, WL + u, DT)),
+                {"text": "global_store_dword %%[loff], v%d, s[%d:%d]%s" % (WL + u, S_WP, S_WP + 1, " offset:%d" % imm if imm else ""), "vm": ("wr", c)},
+                plain("ds_write_b32 %%[scw], v%d%s" % (WL + u, " offset:256" if c & 1 else ""))]
     for i in range(4):
         pro.append(gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0, ("st", 0)))       # chunk 0 of the rotations, through the chunk registers
     pro += neuron_loads(0, 0, 0) + neuron_loads(1, 256, 1)
@@ -77,26 +88,33 @@ def lone_wave_loop(mode):
     pro.append(wait([("st", 0)]))
     for i in range(4):
         pro.append(plain("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else "")))
+    if upd:
+        pro += update(0, 0, 0)
     pro += [plain("s_waitcnt lgkmcnt(0)"), plain("s_barrier"), plain("0:")]
 
     def chunk(u, c):        # chunk c = 4 * pass + u; tags are absolute so that the counting below can find them
         out = []
         rd, wr = (u & 1) * STAGE, ((u + 1) & 1) * STAGE
+        nv = NV if upd else NV + 4 * u
+        if upd:
+            # the chunk's new values in the operand layout, then, unless this is the last chunk, the update of the next
+            out.append(plain("ds_read_b128 %s, %%[scr]%s" % (vr(NV), " offset:256" if u & 1 else "")))
         for q in range(16):
             off = rd + 16 * q
             out.append(plain("ds_read_b128 %s, %%[ldsr]%s" % (vr(BV + 4 * q), " offset:%d" % off if off else "")))
-        nv, xv = NV + 4 * u, XV + 4 * u
-        mine = [("nv", c)] + ([("xv", c)] if upd else [])
-        if store:
+        mine = [("nv", c)]
+        if upd:
+            out += [plain("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1)), plain("s_cbranch_scc1 2f")]
+            out += update((u + 1) & 3, c + 1, (u + 1) * 256)
+            out.append(plain("2:"))
+        elif store:
             out.append(wait(mine))
-            if upd:
-                out += [plain("v_sub_f32_e32 v%d, v%d, v%d" % (DT + r, nv + r, xv + r)) for r in range(4)]
-                out += [plain("v_mul_f32_e32 v%d, s%d, v%d" % (DT + r, S_F, DT + r)) for r in range(4)]
-                out += [plain("v_sub_f32_e32 v%d, v%d, v%d" % (nv + r, nv + r, DT + r)) for r in range(4)]
             out.append({"text": "global_store_dwordx4 %%[noff], %s, s[%d:%d]%s" % (vr(nv), S_WP, S_WP + 1, " offset:%d" % (u * 256) if u else ""),
                         "vm": ("wr", c)})
         for sl in range(4):
-            # (the neuron vector with the first slab; the rotation vectors that go to LDS behind the last slab with it)
+            # (the neuron vector with the first slab; the rotation vectors that go to LDS behind the last slab with it.
+            # UPDATE: 17 or, with the write of the update, 18 LDS operations are in the queue, the neuron's values first:
+            # the counts are those of 17)
             out.append(wait(mine if sl == 0 and not store else [("st", c + 1)] if sl == 3 else [], 12 - 4 * sl))
             def sub(e):
                 return plain("v_sub_f32_dpp v%d, v%d, v%d row_newbcast:%d row_mask:0xf bank_mask:0xf" % (
@@ -107,7 +125,9 @@ def lone_wave_loop(mode):
             for e in range(8):
                 out += [fma(e), sub(8 + e)]
             out += [fma(8 + e) for e in range(8)]
-        out += [plain("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1)), plain("s_cbranch_scc1 1f")]
+        if not upd:
+            out.append(plain("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1)))
+        out.append(plain("s_cbranch_scc1 1f"))           # (UPDATE: the comparison above still stands)
         st = ST[u & 1]
         out += [plain("ds_write_b128 %%[ldsw], %s offset:%d" % (vr(st + 4 * i), wr + i * ROWS16)) for i in range(4)]
         out += [gload(st + 4 * i, "%%[roff%d]" % i, S_RP, (u + 3) * 256, ("st", c + 3)) for i in range(4)]
@@ -156,11 +176,14 @@ def lone_wave_loop(mode):
     A.append("s_waitcnt vmcnt(0)")
 
     name = NAMES[mode]
-    extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f", COPY: ", float *wp"}[mode]
-    extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f)', COPY: ', [wp] "s"(wp)'}[mode]
+    extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f, uint32_t loff, uint32_t scw, uint32_t scr", COPY: ", float *wp"}[mode]
+    extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f), [loff] "v"(loff), [scw] "v"(scw), [scr] "v"(scr)',
+                 COPY: ', [wp] "s"(wp)'}[mode]
     lines = []
     lines.append({PLAIN: "// The chunk loop of the kernel for small problems, one neuron per wave (see gen_ssd_steps.py).",
-                  UPDATE: "// The same loop, the neuron pulled toward the variant row xp with factor f first and its new row stored to wp.",
+                  UPDATE: "// The same loop, the neuron pulled toward the variant row xp with factor f first and its new row stored to wp\n"
+                          "// (loff: byte offset of the lane's element in a chunk; scw, scr: LDS byte addresses of the lane's element and of its\n"
+                          "// 16-byte piece in 512 bytes of the wave's own).",
                   COPY: "// The same loop, the neuron's row also stored to wp as it is."}[mode])
     if mode == PLAIN:
         lines.append("// roff: byte offsets of the thread's four staging vectors in a chunk of the block's 64 rotation rows; noff: byte")
@@ -173,7 +196,7 @@ def lone_wave_loop(mode):
     lines.append('        : [acc] "+v"(acc)')
     lines.append('        : [roff0] "v"(roff0), [roff1] "v"(roff1), [roff2] "v"(roff2), [roff3] "v"(roff3), [noff] "v"(noff), [ldsw] "v"(ldsw),')
     lines.append('          [ldsr] "v"(ldsr), [rp] "s"(rp), [np] "s"(np), [cnt] "s"(chunks)%s' % extra_ops)
-    clob = ['"v%d"' % r for r in range(BV, (XV if upd else NV) + 16)] + ['"s%d"' % r for r in range(S_RP, S_WP + 2)] + ['"scc"', '"memory"']
+    clob = ['"v%d"' % r for r in range(BV, XL + 4 if upd else NV + 16)] + ['"s%d"' % r for r in range(S_RP, S_WP + 2)] + ['"scc"', '"memory"']
     rows = [", ".join(clob[i:i + 16]) for i in range(0, len(clob), 16)]
     lines.append("        : " + ",\n          ".join(rows) + ");")
     lines.append("}")

@@ -696,9 +696,9 @@ __global__ __launch_bounds__(256, 2) void k_dist_f32_dpp(const float *__restrict
 // leaves it.  The update of image i - 1 costs a launch of its own about a third of the distance kernel's time
 // (each of its blocks waits for the keys, searches the best match, then waits for its factor); here every
 // wave applies it to its neuron on the fly instead -- w = w - ((w - x) * f) on each chunk of the neuron's
-// operand row as it arrives, x the same chunk of the row of the variant of image i - 1 that was closest to the
-// neuron -- and stores the new row to the other of two operand buffers (all waves of a neuron store the same
-// bytes; an untouched neuron's row is copied).  What a wave needs for it does not depend on the search: the
+// operand row one chunk ahead of its use, x the same chunk of the row of the variant of image i - 1 that was
+// closest to the neuron -- and stores the new row to the other of two operand buffers (all waves of a neuron
+// store the same bytes; an untouched neuron's row is copied).  What a wave needs for it does not depend on the search: the
 // keys of image i - 1 and the neuron's whole column of the factor matrix are requested together, the best
 // match is the minimum over the wave, the factor comes out of the column by lane.  The neuron's full image
 // (all elements, not only the region that the operand row holds) is not on this path: k_update_replay applies
@@ -716,12 +716,14 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
                                                           uint32_t R, uint32_t Rpad, PrevImage prev)
 {
     __shared__ v4f s_rot[2][64 * kDistRow / 4];
+    __shared__ float s_upd[4][2][64];          // per wave: the updated chunk on its way into the operand layout, two stages
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t r0 = blockIdx.x * kWave;
     const uint32_t n = blockIdx.y * 4 + wave, nc = min(n, N - 1);
     const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
     const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) v4f *)&s_rot[0][0];
+    const uint32_t upd = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)&s_upd[0][0][0];
     const uint32_t roff0 = (lrow * Epad + lcol) * 4, roff1 = ((lrow + 16) * Epad + lcol) * 4,
                    roff2 = ((lrow + 32) * Epad + lcol) * 4, roff3 = ((lrow + 48) * Epad + lcol) * 4;
     const uint32_t noff = (lane & 15) * 16, ldsw = lds + (lrow * kDistRow + lcol) * 4, ldsr = lds + lane * kDistRow * 4;
@@ -778,7 +780,8 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
             ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
         else
             ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks,
-                                      prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad, wp, f);
+                                      prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad, wp, f, lane * 4,
+                                      upd + wave * 512 + lane * 4, upd + wave * 512 + (lane & 15) * 16);
     }
     const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
     if (lane == 0 && n < N) atomicMin(&key[n], kv);
