@@ -750,6 +750,8 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         const v4f warm0 = *(const v4f *)((const char *)rp + roff0), warm1 = *(const v4f *)((const char *)rp + roff1),
                   warm2 = *(const v4f *)((const char *)rp + roff2), warm3 = *(const v4f *)((const char *)rp + roff3),
                   warm4 = *(const v4f *)((const char *)np + noff);
+        // (the compiler would request r where it is used, behind the search: a round trip of its own)
+        asm volatile("" ::"s"(r));
         // The best match: the smallest distance of the wave (a reduction over the lanes by DPP), then the first
         // neuron that has it.
         uint32_t dmin = 0xffffffffu;
