@@ -47,16 +47,16 @@ MEASURED_VALU_LANE_OPS_T = 50.0     # subtract / fma stream, eight waves per SIM
 # by what the same counter reads for a device-to-device copy of known size; (bytes, the summary
 # under profiles/ that holds the readings).  Not measured in the run that prints the line.
 COUNTER_TRAFFIC_PER_IMAGE = {
-    ("cfg0", "distance"): (12.245e6 + 3.264e6, "profiles/cfg0_train_f32_counters.txt"),   # with the update of the image before
-    ("cfg0", "update"): ((27.486e6 + 0.774e6 + 1.590e6 + 1.184e6) / 64, "profiles/cfg0_train_f32_counters.txt"),   # per group of 64
-    ("cfg1", "rotate"): ((95.060e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg1", "distance"): ((214.633e6 + 1.639e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg2", "distance"): (26.958e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (25.150e6 + 20.722e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (876.388e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg0", "distance"): (12.216e6 + 3.239e6, "profiles/cfg0_train_f32_counters.txt"),   # with the update of the image before
+    ("cfg0", "update"): ((18.466e6 + 0.774e6 + 1.712e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
+    ("cfg1", "rotate"): ((95.405e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg1", "distance"): ((214.632e6 + 1.640e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg2", "distance"): (26.944e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (27.029e6 + 20.734e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg3", "distance"): (835.448e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
-    ("cfg3", "update"): (63.762e6 + 47.153e6 + (998.532e6 + 95.565e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg4", "update"): (1.210e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
+    ("cfg3", "update"): (73.958e6 + 47.153e6 + (1000.797e6 + 95.565e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg4", "update"): (1.205e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
 }
 
 # Images per step of the workloads that ride along in `all_configs` (the headline workload always
@@ -255,7 +255,7 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
                  "published 157.3 TFLOP/s is this form's ceiling" % MEASURED_VALU_LANE_OPS_T)
         if w.mode == "train" and 0 < times["update"][0] < times["distance"][0]:
             notes += ("; a small float32 trainer: the distance launch of an image also applies the update of the image "
-                      "before it to the SOM operand (per chunk of 64 elements 14 instructions next to the 128 of the "
+                      "before it to the SOM operand (per chunk of 64 elements 8 instructions next to the 128 of the "
                       "distances, not counted as operations), so the launch priced here is the whole step of an image "
                       "but for one launch per group that brings the neurons' full images up to date")
     elif dominant == "distance" and path in (capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA_GEMM, capi.KERNEL_MFMA):
