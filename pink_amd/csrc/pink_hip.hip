@@ -711,6 +711,7 @@ struct PrevImage {
     uint32_t *bmu_out, *counts;
 };
 
+template <int NQ>     // neurons / 64, rounded up: keys and factors per lane in the search
 __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                           unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
                                                           uint32_t R, uint32_t Rpad, PrevImage prev)
@@ -733,13 +734,13 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
     if (prev.key == nullptr) {
         ssd_lone_wave_loop(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks);
     } else {
-        // (N <= 256: four keys and four factors per lane; every load is issued before the first is used, indices
+        // (NQ keys and NQ factors per lane; every load is issued before the first is used, indices
         // past the end are clamped and dropped afterwards)
         const uint32_t *key32 = (const uint32_t *)prev.key;          // little endian: rotation, then the distance bits
-        uint32_t dist[4];
-        float fcol[4];
+        uint32_t dist[NQ];
+        float fcol[NQ];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < NQ; ++q) {
             const uint32_t m = min(lane + 64 * q, N - 1);
             dist[q] = key32[2 * m + 1];
             fcol[q] = prev.factors_t[(size_t)nc * N + m];
@@ -756,7 +757,7 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         // neuron that has it.
         uint32_t dmin = 0xffffffffu;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < NQ; ++q) {
             if (lane + 64 * q >= N) dist[q] = 0xffffffffu;
             dmin = min(dmin, dist[q]);
         }
@@ -764,7 +765,7 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         uint32_t bmu = 0;
         float f = 0.0f;
 #pragma unroll
-        for (int q = 3; q >= 0; --q) {
+        for (int q = NQ - 1; q >= 0; --q) {
             const unsigned long long hit = __ballot(dist[q] == best && lane + 64 * q < N);
             if (hit) {
                 const uint32_t at = (uint32_t)__builtin_ctzll(hit);
@@ -2215,9 +2216,12 @@ int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu
         prev.bmu_out = bmu_prev;
         prev.counts = ctx->d_counts;
     }
-    hipLaunchKernelGGL(k_train_f32_dpp, dim3(ctx->Rpad / kWave, (ctx->N + 3) / 4), dim3(256), 0, ctx->stream,
-                       (const float *)ctx->d_somP, (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad,
-                       ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, prev);
+#define LAUNCH_TRAIN_F32(NQ_)                                                                                          \
+    hipLaunchKernelGGL(k_train_f32_dpp<NQ_>, dim3(ctx->Rpad / kWave, (ctx->N + 3) / 4), dim3(256), 0, ctx->stream,      \
+                       (const float *)ctx->d_somP, (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad,   \
+                       ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, prev)
+    if (ctx->N <= 128) LAUNCH_TRAIN_F32(2); else LAUNCH_TRAIN_F32(4);
+#undef LAUNCH_TRAIN_F32
     if (has_prev) std::swap(ctx->d_somP, ctx->d_somP_alt);        // the updated operand is the current one now
     return launch_check(ctx, "k_train_f32_dpp");
 }
@@ -2792,7 +2796,10 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
         }
-        // one launch per image where the float32 distance kernel runs in its one-wave-per-SIMD form (see k_train_f32_dpp)
+        // one launch per image where the float32 distance kernel runs in its one-wave-per-SIMD form (see k_train_f32_dpp;
+        // up to 256 neurons: measured with 512 allowed, 17 x 17 and 18 x 18 neurons at 720 variants train no faster this
+        // way than with an update launch of their own -- with three to four waves per SIMD the launch saved is paid in
+        // instructions)
         ctx->fused_f32_train = c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv && ctx->N <= 256 &&
                                (size_t)(ctx->Rpad / kWave) * ((ctx->N + 3) / 4) <= (size_t)4 * ctx->num_cu;
         ctx->rows_f32_train = !ctx->fused_f32_train && c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv &&
