@@ -72,3 +72,12 @@ def test_synthetic_images_are_deterministic_and_in_range():
         b = synthetic.images(w, 5)
         assert np.array_equal(a, b)
         assert a.min() >= 0.0 and a.max() <= 1.0 and a.dtype == np.float32
+
+
+def test_generated_assembly_loop_is_current():
+    # pink_amd/csrc/ssd_steps.inc is what gen_ssd_steps.py writes: the build compiles the committed file
+    import subprocess, sys
+    csrc = os.path.join(ROOT, "pink_amd", "csrc")
+    out = subprocess.run([sys.executable, os.path.join(csrc, "gen_ssd_steps.py")], check=True, capture_output=True, text=True).stdout
+    with open(os.path.join(csrc, "ssd_steps.inc")) as f:
+        assert f.read() == out
