@@ -30,7 +30,10 @@ def lone_wave_loop(mode):
 
     Element e of a chunk of the neuron sits in register e % 4 of lane e / 4 of every row of 16 lanes (one
     16-byte load per lane) and reaches all lanes of the row as the DPP operand of the subtract; every
-    (neuron, rotation) sum is one lane's multiply-add chain in element order.
+    (neuron, rotation) sum is one lane's multiply-add chain in element order.  A DPP operand must not be read within
+    two instruction slots of a vector-ALU write of its register (nothing checks that inside assembly): in all three
+    forms the registers that the subtracts read through DPP are written by memory or LDS loads only, behind counted
+    waits, never by the vector ALU.
 
     Three forms.  PLAIN computes the distances.  UPDATE first pulls the neuron toward a variant x with factor
     f -- w = w - ((w - x) * f), three roundings -- stores the new row to a second buffer and computes the distances
