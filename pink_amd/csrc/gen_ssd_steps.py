@@ -81,18 +81,29 @@ def lone_wave_loop(mode):
                 plain("v_sub_f32_e32 v%d, v%d, v%d" % (WL + u, WL + u, DT)),
                 {"text": "global_store_dword %%[loff], v%d, s[%d:%d]%s" % (WL + u, S_WP, S_WP + 1, " offset:%d" % imm if imm else ""), "vm": ("wr", c)},
                 plain("ds_write_b32 %%[scw], v%d%s" % (WL + u, " offset:256" if c & 1 else ""))]
-    for i in range(4):
-        pro.append(gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0, ("st", 0)))       # chunk 0 of the rotations, through the chunk registers
-    pro += neuron_loads(0, 0, 0) + neuron_loads(1, 256, 1)
+    if upd:
+        # The caller has chunk 0 of the rotations in LDS already and brings chunk 0 of the neuron and of the variant in
+        # registers (it requested them ahead of its search for the best match, whose result this form needs): what is
+        # left of the prologue is the requests that run ahead and the update of chunk 0.
+        pro += neuron_loads(1, 256, 1)
+    else:
+        for i in range(4):
+            pro.append(gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0, ("st", 0)))   # chunk 0 of the rotations, through the chunk registers
+        pro += neuron_loads(0, 0, 0) + neuron_loads(1, 256, 1)
     pro += [gload(ST[0] + 4 * i, "%%[roff%d]" % i, S_RP, 256, ("st", 1)) for i in range(4)]
     pro += neuron_loads(2, 512, 2)
     pro += [gload(ST[1] + 4 * i, "%%[roff%d]" % i, S_RP, 512, ("st", 2)) for i in range(4)]
     pro += neuron_loads(3, 768, 3)
-    pro.append(wait([("st", 0)]))
-    for i in range(4):
-        pro.append(plain("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else "")))
     if upd:
-        pro += update(0, 0, 0)
+        pro += [plain("v_sub_f32_e32 v%d, %%[w0], %%[x0]" % XL),               # (register set 0 is free until chunk 4 is requested)
+                plain("v_mul_f32_e32 v%d, s%d, v%d" % (XL, S_F, XL)),
+                plain("v_sub_f32_e32 v%d, %%[w0], v%d" % (WL, XL)),
+                {"text": "global_store_dword %%[loff], v%d, s[%d:%d]" % (WL, S_WP, S_WP + 1), "vm": ("wr", 0)},
+                plain("ds_write_b32 %%[scw], v%d" % WL)]
+    else:
+        pro.append(wait([("st", 0)]))
+        for i in range(4):
+            pro.append(plain("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else "")))
     pro += [plain("s_waitcnt lgkmcnt(0)"), plain("s_barrier"), plain("0:")]
 
     def chunk(u, c):        # chunk c = 4 * pass + u; tags are absolute so that the counting below can find them
@@ -179,14 +190,16 @@ def lone_wave_loop(mode):
     A.append("s_waitcnt vmcnt(0)")
 
     name = NAMES[mode]
-    extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f, uint32_t loff, uint32_t scw, uint32_t scr", COPY: ", float *wp"}[mode]
-    extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f), [loff] "v"(loff), [scw] "v"(scw), [scr] "v"(scr)',
+    extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f, uint32_t loff, uint32_t scw, uint32_t scr, float w0, float x0",
+                  COPY: ", float *wp"}[mode]
+    extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f), [loff] "v"(loff), [scw] "v"(scw), [scr] "v"(scr), [w0] "v"(w0), [x0] "v"(x0)',
                  COPY: ', [wp] "s"(wp)'}[mode]
     lines = []
     lines.append({PLAIN: "// The chunk loop of the kernel for small problems, one neuron per wave (see gen_ssd_steps.py).",
                   UPDATE: "// The same loop, the neuron pulled toward the variant row xp with factor f first and its new row stored to wp\n"
                           "// (loff: byte offset of the lane's element in a chunk; scw, scr: LDS byte addresses of the lane's element and of its\n"
-                          "// 16-byte piece in 512 bytes of the wave's own).",
+                          "// 16-byte piece in 512 bytes of the wave's own; w0, x0: the lane's element of chunk 0 of the neuron and of the variant.\n"
+                          "// The caller has stored chunk 0 of the rotation rows to LDS stage 0; the loop's first barrier publishes it.)",
                   COPY: "// The same loop, the neuron's row also stored to wp as it is."}[mode])
     if mode == PLAIN:
         lines.append("// roff: byte offsets of the thread's four staging vectors in a chunk of the block's 64 rotation rows; noff: byte")

@@ -746,13 +746,13 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
             fcol[q] = prev.factors_t[(size_t)nc * N + m];
         }
         const uint32_t r = key32[2 * nc];                            // the neuron's closest variant of image i - 1
-        // (the loop's first requests, made here as well: they travel while the search below runs, and the loop
-        // finds the lines near)
-        const v4f warm0 = *(const v4f *)((const char *)rp + roff0), warm1 = *(const v4f *)((const char *)rp + roff1),
-                  warm2 = *(const v4f *)((const char *)rp + roff2), warm3 = *(const v4f *)((const char *)rp + roff3),
-                  warm4 = *(const v4f *)((const char *)np + noff);
-        // (the compiler would request r where it is used, behind the search: a round trip of its own)
-        asm volatile("" ::"s"(r));
+        // Chunk 0 of the rotation rows, of the neuron and (as soon as r is there) of the variant are requested here,
+        // ahead of the search: they travel while it runs, go to LDS stage 0 and to the loop as registers behind it.
+        const v4f first0 = *(const v4f *)((const char *)rp + roff0), first1 = *(const v4f *)((const char *)rp + roff1),
+                  first2 = *(const v4f *)((const char *)rp + roff2), first3 = *(const v4f *)((const char *)rp + roff3);
+        const float w0 = np[lane];
+        const float *xp = prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad;
+        const float x0 = xp[lane];
         // The best match: the smallest distance of the wave (a reduction over the lanes by DPP), then the first
         // neuron that has it.
         uint32_t dmin = 0xffffffffu;
@@ -777,14 +777,16 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
             *prev.bmu_out = bmu;
             atomicAdd(&prev.counts[bmu], 1u);          // m_update_info[bmu]++ (Trainer.h:302-303)
         }
-        asm volatile("" ::"v"(warm0), "v"(warm1), "v"(warm2), "v"(warm3), "v"(warm4));
         float *wp = prev.somP_next + (size_t)nc * Epad;
-        if (f == 0.0f)
+        if (f == 0.0f) {
+            asm volatile("" ::"v"(first0), "v"(first1), "v"(first2), "v"(first3), "v"(w0), "v"(x0));   // (requested, not used)
             ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
-        else
-            ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks,
-                                      prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad, wp, f, lane * 4,
-                                      upd + wave * 512 + lane * 4, upd + wave * 512 + (lane & 15) * 16);
+        } else {
+            v4f *stage0 = &s_rot[0][(lrow * kDistRow + lcol) / 4];
+            stage0[0] = first0; stage0[16 * kDistRow / 4] = first1; stage0[32 * kDistRow / 4] = first2; stage0[48 * kDistRow / 4] = first3;
+            ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, xp, wp, f, lane * 4,
+                                      upd + wave * 512 + lane * 4, upd + wave * 512 + (lane & 15) * 16, w0, x0);
+        }
     }
     const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
     if (lane == 0 && n < N) atomicMin(&key[n], kv);
