@@ -23,7 +23,7 @@ def lone_wave_loop(mode):
     """The whole chunk loop of the kernel for small problems (one neuron per wave, about one wave per SIMD) as
     ONE asm statement.  A lone wave issues an instruction of any kind about every eight clocks, so the loop is
     written down to the instruction: per 64-element chunk 64 DPP subtracts, 64 multiply-adds, 16 LDS reads,
-    4 LDS writes, 5 global loads, 5 waits, a barrier and a compare-and-branch.  It is assembly as a whole
+    4 LDS writes, 5 global loads, 3 waits, a barrier and a compare-and-branch.  It is assembly as a whole
     because its loads run three and four chunks ahead with counted waits: the compiler neither keeps such
     loads where they are written nor knows, for loads issued by assembly, that a register is still being
     written -- inside one statement with fixed registers there is nothing for it to move, copy or reuse.
@@ -126,10 +126,16 @@ def lone_wave_loop(mode):
             out.append({"text": "global_store_dwordx4 %%[noff], %s, s[%d:%d]%s" % (vr(nv), S_WP, S_WP + 1, " offset:%d" % (u * 256) if u else ""),
                         "vm": ("wr", c)})
         for sl in range(4):
-            # (the neuron vector with the first slab; the rotation vectors that go to LDS behind the last slab with it.
-            # UPDATE: 17 or, with the write of the update, 18 LDS operations are in the queue, the neuron's values first:
-            # the counts are those of 17)
-            out.append(wait(mine if sl == 0 and not store else [("st", c + 1)] if sl == 3 else [], 12 - 4 * sl))
+            # Two waits for the chunk's LDS reads: the first slab's before it (with the neuron vector where it comes from
+            # memory), everything else before the second -- by then the first slab's 32 instructions have given the
+            # other reads all the time they need, so a wait per slab would only cost its instruction slot; the rotation
+            # vectors that go to LDS behind the last slab, requested two chunks ago, ride on the second wait.
+            # (UPDATE: 17 or, with the write of the update, 18 LDS operations are in the queue, the neuron's values
+            # first: the first count is that of 17.)
+            if sl == 0:
+                out.append(wait(mine if not store else [], 12))
+            elif sl == 1:
+                out.append(wait([("st", c + 1)], 0))
             def sub(e):
                 return plain("v_sub_f32_dpp v%d, v%d, v%d row_newbcast:%d row_mask:0xf bank_mask:0xf" % (
                     DT + (e & 7), nv + (e & 3), BV + 16 * sl + e, 4 * sl + e // 4))
