@@ -53,9 +53,9 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg1", "distance"): ((214.632e6 + 1.640e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg2", "distance"): (26.944e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
     ("cfg2", "update"): (27.029e6 + 20.734e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (835.448e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "distance"): (874.783e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
-    ("cfg3", "update"): (73.958e6 + 47.153e6 + (1000.797e6 + 95.565e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "update"): (73.898e6 + 47.153e6 + (294.770e6 + 94.546e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
     ("cfg4", "update"): (1.205e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
 }
 

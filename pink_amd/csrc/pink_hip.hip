@@ -1411,7 +1411,9 @@ __global__ __launch_bounds__(256) void k_update_replay(float *__restrict__ som, 
 {
     __shared__ float s_f[kReplayMax];
     __shared__ uint32_t s_row[kReplayMax];   // stored row of the group's variants * 4 + how it is read
-    const uint32_t n = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
+    // (neurons vary fastest over the grid: the blocks that run side by side then read the same stretch of elements of
+    // whatever variants their neurons were closest to -- a few MB that stay in L2 -- and not whole variants)
+    const uint32_t n = blockIdx.x, j = blockIdx.y * 256 + threadIdx.x;
     if (threadIdx.x < images) {
         const uint32_t i = threadIdx.x;
         const uint32_t r = (uint32_t)(key[(size_t)i * N + n] & ((1ull << shift) - 1ull));
@@ -2250,7 +2252,7 @@ int run_update_replay(pink_hip_ctx *ctx, uint32_t images, const uint32_t *dev_bm
     if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
     for (uint32_t first = 0; first < images; first += kReplayMax) {
         const uint32_t count = std::min(kReplayMax, images - first);
-        hipLaunchKernelGGL(k_update_replay, dim3((ctx->S + 255) / 256, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,
+        hipLaunchKernelGGL(k_update_replay, dim3(ctx->N, (ctx->S + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_som,
                            ctx->d_rot + (size_t)first * ctx->R * ctx->S, ctx->d_key + (size_t)first * ctx->N, ctx->d_factors,
                            dev_bmu + first, count, ctx->N, ctx->S, ctx->R, ctx->shift, vp);
         TRY(launch_check(ctx, "k_update_replay"));
