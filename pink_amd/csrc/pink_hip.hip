@@ -3131,9 +3131,9 @@ hipError_t stage_in(pink_hip_ctx *ctx, void *dev, const void *host, size_t bytes
 }
 
 // `n` host images into the staging buffer and through `run(device images, first image, count)`,
-// in pieces of about 64 MB: the copy of a piece goes over a second stream while the kernels of the
-// piece before it run (also from pageable memory, where the copy call returns when the piece has
-// left the host buffer).  Small inputs take the pinned bounce buffer in one go.
+// in pieces that grow from about 1 MB to 16 or 64 MB: the copy of a piece goes over a second stream
+// while the kernels of the piece before it run (also from pageable memory, where the copy call
+// returns when the piece has left the host buffer).  Small inputs take the pinned bounce buffer in one go.
 extern "C++" {
 template <typename Run>
 int staged_run(pink_hip_ctx *ctx, const float *host_images, uint32_t n, Run run)
@@ -3152,11 +3152,17 @@ int staged_run(pink_hip_ctx *ctx, const float *host_images, uint32_t n, Run run)
     ctx->st_ring_busy = false;
     // (a trainer's kernels take long enough per image for 16 MB pieces to hide all copies but the first behind them:
     // cfg0 40 k -> 51 k images/s with pageable buffers; a mapper's launch groups want the larger pieces)
-    uint32_t piece = (uint32_t)std::max<size_t>(1, ((size_t)(ctx->trainer ? 16 : 64) << 20) / img_bytes);
-    if (piece > ctx->Bcap) piece -= piece % ctx->Bcap;     // whole launch groups
-    uint32_t turn = 0;
-    for (uint32_t first = 0; first < n; first += piece, turn ^= 1) {
-        const uint32_t count = std::min(piece, n - first);
+    // Nothing hides the copy of the first piece, so the pieces start at about 1 MB and double up to that size.
+    const auto whole_groups = [&](size_t bytes) {
+        uint32_t images = (uint32_t)std::max<size_t>(1, bytes / img_bytes);
+        if (images > ctx->Bcap) images -= images % ctx->Bcap;
+        return images;
+    };
+    const uint32_t largest = whole_groups((size_t)(ctx->trainer ? 16 : 64) << 20);
+    uint32_t piece = std::min(largest, std::max(whole_groups((size_t)1 << 20), std::min(ctx->Bcap, largest)));
+    uint32_t turn = 0, count = 0;
+    for (uint32_t first = 0; first < n; first += count, turn ^= 1, piece = std::min(largest, 2 * piece)) {
+        count = std::min(piece, n - first);
         float *dev = ctx->st_img + (size_t)first * ctx->isz;
         HIP_TRY(ctx, hipMemcpyAsync(dev, host_images + (size_t)first * ctx->isz, count * img_bytes, hipMemcpyHostToDevice,
                                     ctx->copy_stream));

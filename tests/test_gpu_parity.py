@@ -338,6 +338,8 @@ SYM_SHAPES = [
     (130, 1, 64, 64, 360, True, 44, capi.CIRCULAR, 2),     # wide form, 48 k-steps, nine slices
     (9, 1, 52, 42, 360, True, 38, capi.QUADRATIC, 40),     # wide form, several images per group
     (20, 2, 40, 30, 360, False, 30, capi.QUADRATIC, 4),    # wide form, two channels, no flip
+    (40, 1, 24, 18, 40, True, 16, capi.QUADRATIC, 600),    # ten column tiles: a whole block and two tiles for the kernel that splits k, more images than its blocks
+    (100, 1, 45, 32, 72, True, 27, capi.QUADRATIC, 5),     # 25 column tiles at 24 k-steps: three blocks and one tile
 ]
 
 
