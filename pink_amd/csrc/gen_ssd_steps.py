@@ -19,7 +19,7 @@ PLAIN, UPDATE, COPY = 0, 1, 2
 NAMES = {PLAIN: "ssd_lone_wave_loop", UPDATE: "ssd_lone_wave_loop_update", COPY: "ssd_lone_wave_loop_copy"}
 
 
-def lone_wave_loop(mode):
+def lone_wave_loop(mode, stage=True):
     """The whole chunk loop of the kernel for small problems (one neuron per wave, about one wave per SIMD) as
     ONE asm statement.  A lone wave issues an instruction of any kind about every eight clocks, so the loop is
     written down to the instruction: per 64-element chunk 64 DPP subtracts, 64 multiply-adds, 16 LDS reads,
@@ -50,7 +50,10 @@ def lone_wave_loop(mode):
     order of issue, so "at most n outstanding" waits for everything but the last n: the n of every wait is
     counted below over the prologue and three passes of the loop, the smallest count of a place is the one
     that holds in all of them (a smaller n waits for older operations too, which by then have long arrived).
-    The last chunk issues no loads; the loads of the three chunks before it read past the end of the rows."""
+    The last chunk issues no loads; the loads of the three chunks before it read past the end of the rows.
+
+    stage=False: the same three forms for a fifth or sixth wave of a block, which computes its neuron against the
+    rotation rows that the first four put into LDS and moves none of them itself (same barriers)."""
     upd, store = mode == UPDATE, mode != PLAIN
     def vr(base, n=4):
         return "v[%d:%d]" % (base, base + n - 1)
@@ -62,8 +65,8 @@ def lone_wave_loop(mode):
     def wait(tags, lgkm=None):
         return {"wait": tags, "lgkm": lgkm}
 
-    pro = [plain("s_mov_b64 s[%d:%d], %%[rp]" % (S_RP, S_RP + 1)), plain("s_mov_b64 s[%d:%d], %%[np]" % (S_NP, S_NP + 1)),
-           plain("s_mov_b32 s%d, %%[cnt]" % S_CNT)]
+    pro = ([plain("s_mov_b64 s[%d:%d], %%[rp]" % (S_RP, S_RP + 1))] if stage else []) + [
+           plain("s_mov_b64 s[%d:%d], %%[np]" % (S_NP, S_NP + 1)), plain("s_mov_b32 s%d, %%[cnt]" % S_CNT)]
     if upd:
         pro += [plain("s_mov_b64 s[%d:%d], %%[xp]" % (S_XP, S_XP + 1)), plain("s_mov_b32 s%d, %%[f]" % S_F)]
     if store:
@@ -87,12 +90,14 @@ def lone_wave_loop(mode):
         # left of the prologue is the requests that run ahead and the update of chunk 0.
         pro += neuron_loads(1, 256, 1)
     else:
-        for i in range(4):
+        for i in range(4 if stage else 0):
             pro.append(gload(BV + 4 * i, "%%[roff%d]" % i, S_RP, 0, ("st", 0)))   # chunk 0 of the rotations, through the chunk registers
         pro += neuron_loads(0, 0, 0) + neuron_loads(1, 256, 1)
-    pro += [gload(ST[0] + 4 * i, "%%[roff%d]" % i, S_RP, 256, ("st", 1)) for i in range(4)]
+    if stage:
+        pro += [gload(ST[0] + 4 * i, "%%[roff%d]" % i, S_RP, 256, ("st", 1)) for i in range(4)]
     pro += neuron_loads(2, 512, 2)
-    pro += [gload(ST[1] + 4 * i, "%%[roff%d]" % i, S_RP, 512, ("st", 2)) for i in range(4)]
+    if stage:
+        pro += [gload(ST[1] + 4 * i, "%%[roff%d]" % i, S_RP, 512, ("st", 2)) for i in range(4)]
     pro += neuron_loads(3, 768, 3)
     if upd:
         pro += [plain("v_sub_f32_e32 v%d, %%[w0], %%[x0]" % XL),               # (register set 0 is free until chunk 4 is requested)
@@ -100,7 +105,7 @@ def lone_wave_loop(mode):
                 plain("v_sub_f32_e32 v%d, %%[w0], v%d" % (WL, XL)),
                 {"text": "global_store_dword %%[loff], v%d, s[%d:%d]" % (WL, S_WP, S_WP + 1), "vm": ("wr", 0)},
                 plain("ds_write_b32 %%[scw], v%d" % WL)]
-    else:
+    elif stage:
         pro.append(wait([("st", 0)]))
         for i in range(4):
             pro.append(plain("ds_write_b128 %%[ldsw], %s%s" % (vr(BV + 4 * i), " offset:%d" % (i * ROWS16) if i else "")))
@@ -135,7 +140,7 @@ def lone_wave_loop(mode):
             if sl == 0:
                 out.append(wait(mine if not store else [], 12))
             elif sl == 1:
-                out.append(wait([("st", c + 1)], 0))
+                out.append(wait([("st", c + 1)] if stage else [], 0))
             def sub(e):
                 return plain("v_sub_f32_dpp v%d, v%d, v%d row_newbcast:%d row_mask:0xf bank_mask:0xf" % (
                     DT + (e & 7), nv + (e & 3), BV + 16 * sl + e, 4 * sl + e // 4))
@@ -149,8 +154,9 @@ def lone_wave_loop(mode):
             out.append(plain("s_cmp_eq_u32 s%d, %d" % (S_CNT, u + 1)))
         out.append(plain("s_cbranch_scc1 1f"))           # (UPDATE: the comparison above still stands)
         st = ST[u & 1]
-        out += [plain("ds_write_b128 %%[ldsw], %s offset:%d" % (vr(st + 4 * i), wr + i * ROWS16)) for i in range(4)]
-        out += [gload(st + 4 * i, "%%[roff%d]" % i, S_RP, (u + 3) * 256, ("st", c + 3)) for i in range(4)]
+        if stage:
+            out += [plain("ds_write_b128 %%[ldsw], %s offset:%d" % (vr(st + 4 * i), wr + i * ROWS16)) for i in range(4)]
+            out += [gload(st + 4 * i, "%%[roff%d]" % i, S_RP, (u + 3) * 256, ("st", c + 3)) for i in range(4)]
         out += neuron_loads(u, (u + 4) * 256, c + 4)
         out += [plain("s_waitcnt lgkmcnt(0)"), plain("s_barrier")]
         return out
@@ -188,14 +194,14 @@ def lone_wave_loop(mode):
         for k, item in enumerate(chunk(u, u)):
             A.append(wait_text(item, (u, k)) if "wait" in item else item["text"])
     A.append("s_sub_u32 s%d, s%d, 4" % (S_CNT, S_CNT))
-    for sb in [S_RP, S_NP] + ([S_XP] if upd else []) + ([S_WP] if store else []):
+    for sb in ([S_RP] if stage else []) + [S_NP] + ([S_XP] if upd else []) + ([S_WP] if store else []):
         A.append("s_add_u32 s%d, s%d, 0x400" % (sb, sb))
         A.append("s_addc_u32 s%d, s%d, 0" % (sb + 1, sb + 1))
     A.append("s_branch 0b")
     A.append("1:")
     A.append("s_waitcnt vmcnt(0)")
 
-    name = NAMES[mode]
+    name = NAMES[mode] + ("" if stage else "_unstaged")
     extra_args = {PLAIN: "", UPDATE: ", const float *xp, float *wp, float f, uint32_t loff, uint32_t scw, uint32_t scr, float w0, float x0",
                   COPY: ", float *wp"}[mode]
     extra_ops = {PLAIN: "", UPDATE: ', [xp] "s"(xp), [wp] "s"(wp), [f] "s"(f), [loff] "v"(loff), [scw] "v"(scw), [scr] "v"(scr), [w0] "v"(w0), [x0] "v"(x0)',
@@ -211,13 +217,21 @@ def lone_wave_loop(mode):
         lines.append("// roff: byte offsets of the thread's four staging vectors in a chunk of the block's 64 rotation rows; noff: byte")
         lines.append("// offset of the lane's neuron vector in a chunk; ldsw, ldsr: LDS byte addresses of the thread's first staging")
         lines.append("// vector and of the lane's row in stage 0; rp, np: chunk 0 of the rotation rows and of the neuron row; chunks >= 1.")
-    lines.append("__device__ __forceinline__ void %s(float &acc, uint32_t roff0, uint32_t roff1, uint32_t roff2, uint32_t roff3," % name)
-    lines.append("        uint32_t noff, uint32_t ldsw, uint32_t ldsr, const float *rp, const float *np, uint32_t chunks%s)" % extra_args)
+    if stage:
+        lines.append("__device__ __forceinline__ void %s(float &acc, uint32_t roff0, uint32_t roff1, uint32_t roff2, uint32_t roff3," % name)
+        lines.append("        uint32_t noff, uint32_t ldsw, uint32_t ldsr, const float *rp, const float *np, uint32_t chunks%s)" % extra_args)
+    else:
+        lines = ["// %s for a wave that stages no rotation rows (the block's first four do): the same operands but for" % NAMES[mode],
+                 "// roff, ldsw and rp; UPDATE: the caller stores nothing to LDS."]
+        lines.append("__device__ __forceinline__ void %s(float &acc, uint32_t noff, uint32_t ldsr, const float *np, uint32_t chunks%s)" % (name, extra_args))
     lines.append("{")
     lines.append("    asm volatile(" + "\n        ".join('"%s\\n\\t"' % a for a in A))
     lines.append('        : [acc] "+v"(acc)')
-    lines.append('        : [roff0] "v"(roff0), [roff1] "v"(roff1), [roff2] "v"(roff2), [roff3] "v"(roff3), [noff] "v"(noff), [ldsw] "v"(ldsw),')
-    lines.append('          [ldsr] "v"(ldsr), [rp] "s"(rp), [np] "s"(np), [cnt] "s"(chunks)%s' % extra_ops)
+    if stage:
+        lines.append('        : [roff0] "v"(roff0), [roff1] "v"(roff1), [roff2] "v"(roff2), [roff3] "v"(roff3), [noff] "v"(noff), [ldsw] "v"(ldsw),')
+        lines.append('          [ldsr] "v"(ldsr), [rp] "s"(rp), [np] "s"(np), [cnt] "s"(chunks)%s' % extra_ops)
+    else:
+        lines.append('        : [noff] "v"(noff), [ldsr] "v"(ldsr), [np] "s"(np), [cnt] "s"(chunks)%s' % extra_ops)
     clob = ['"v%d"' % r for r in range(BV, XL + 4 if upd else NV + 16)] + ['"s%d"' % r for r in range(S_RP, S_WP + 2)] + ['"scc"', '"memory"']
     rows = [", ".join(clob[i:i + 16]) for i in range(0, len(clob), 16)]
     lines.append("        : " + ",\n          ".join(rows) + ");")
@@ -226,6 +240,7 @@ def lone_wave_loop(mode):
 
 
 print("// Generated by gen_ssd_steps.py -- do not edit.")
-for mode in (PLAIN, UPDATE, COPY):
-    print()
-    print(lone_wave_loop(mode))
+for stage in (True, False):
+    for mode in (PLAIN, UPDATE, COPY):
+        print()
+        print(lone_wave_loop(mode, stage))

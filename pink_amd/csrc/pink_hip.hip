@@ -712,17 +712,21 @@ struct PrevImage {
 };
 
 template <int NQ>     // neurons / 64, rounded up: keys and factors per lane in the search
-__global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
+__global__ __launch_bounds__(384) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                           unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
                                                           uint32_t R, uint32_t Rpad, PrevImage prev)
 {
     __shared__ v4f s_rot[2][64 * kDistRow / 4];
-    __shared__ float s_upd[4][2][64];          // per wave: the updated chunk on its way into the operand layout, two stages
+    __shared__ float s_upd[6][2][64];          // per wave: the updated chunk on its way into the operand layout, two stages
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t r0 = blockIdx.x * kWave;
-    const uint32_t n = blockIdx.y * 4 + wave, nc = min(n, N - 1);
-    const uint32_t lrow = tid >> 4, lcol = (tid & 15) * 4;
+    // Four, five or six waves = neurons per block.  The first four move the rotation rows; a fifth and sixth only
+    // compute (where four neurons per block would make more blocks than the chip has CUs and fewer neurons per block
+    // fewer, a CU with two blocks sets the pace for all: better every CU with one block and one or two SIMDs shared).
+    const bool stages = wave < 4;
+    const uint32_t n = blockIdx.y * (blockDim.x >> 6) + wave, nc = min(n, N - 1);
+    const uint32_t lrow = (tid & 255) >> 4, lcol = (tid & 15) * 4;
     const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) v4f *)&s_rot[0][0];
     const uint32_t upd = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) float *)&s_upd[0][0][0];
     const uint32_t roff0 = (lrow * Epad + lcol) * 4, roff1 = ((lrow + 16) * Epad + lcol) * 4,
@@ -732,7 +736,8 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
     const uint32_t chunks = Epad / kDistKC;
     float acc = 0.0f;
     if (prev.key == nullptr) {
-        ssd_lone_wave_loop(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks);
+        if (stages) ssd_lone_wave_loop(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks);
+        else ssd_lone_wave_loop_unstaged(acc, noff, ldsr, np, chunks);
     } else {
         // (NQ keys and NQ factors per lane; every load is issued before the first is used, indices
         // past the end are clamped and dropped afterwards)
@@ -748,8 +753,11 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         const uint32_t r = key32[2 * nc];                            // the neuron's closest variant of image i - 1
         // Chunk 0 of the rotation rows, of the neuron and (as soon as r is there) of the variant are requested here,
         // ahead of the search: they travel while it runs, go to LDS stage 0 and to the loop as registers behind it.
-        const v4f first0 = *(const v4f *)((const char *)rp + roff0), first1 = *(const v4f *)((const char *)rp + roff1),
-                  first2 = *(const v4f *)((const char *)rp + roff2), first3 = *(const v4f *)((const char *)rp + roff3);
+        v4f first0 = {}, first1 = {}, first2 = {}, first3 = {};
+        if (stages) {
+            first0 = *(const v4f *)((const char *)rp + roff0); first1 = *(const v4f *)((const char *)rp + roff1);
+            first2 = *(const v4f *)((const char *)rp + roff2); first3 = *(const v4f *)((const char *)rp + roff3);
+        }
         const float w0 = np[lane];
         const float *xp = prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad;
         const float x0 = xp[lane];
@@ -780,12 +788,16 @@ __global__ __launch_bounds__(256, 2) void k_train_f32_dpp(const float *__restric
         float *wp = prev.somP_next + (size_t)nc * Epad;
         if (f == 0.0f) {
             asm volatile("" ::"v"(first0), "v"(first1), "v"(first2), "v"(first3), "v"(w0), "v"(x0));   // (requested, not used)
-            ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
-        } else {
+            if (stages) ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
+            else ssd_lone_wave_loop_copy_unstaged(acc, noff, ldsr, np, chunks, wp);
+        } else if (stages) {
             v4f *stage0 = &s_rot[0][(lrow * kDistRow + lcol) / 4];
             stage0[0] = first0; stage0[16 * kDistRow / 4] = first1; stage0[32 * kDistRow / 4] = first2; stage0[48 * kDistRow / 4] = first3;
             ssd_lone_wave_loop_update(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, xp, wp, f, lane * 4,
                                       upd + wave * 512 + lane * 4, upd + wave * 512 + (lane & 15) * 16, w0, x0);
+        } else {
+            ssd_lone_wave_loop_update_unstaged(acc, noff, ldsr, np, chunks, xp, wp, f, lane * 4, upd + wave * 512 + lane * 4,
+                                               upd + wave * 512 + (lane & 15) * 16, w0, x0);
         }
     }
     const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
@@ -2220,8 +2232,14 @@ int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu
         prev.bmu_out = bmu_prev;
         prev.counts = ctx->d_counts;
     }
+    // neurons (waves) per block: four, or the five or six that make the launch one block per CU where four do not
+    const uint32_t rblocks = ctx->Rpad / kWave;
+    uint32_t per_block = 4;
+    if (rblocks * ((ctx->N + 3) / 4) > (uint32_t)ctx->num_cu)
+        for (uint32_t w = 5; w <= 6 && per_block == 4; ++w)
+            if (rblocks * ((ctx->N + w - 1) / w) <= (uint32_t)ctx->num_cu) per_block = w;
 #define LAUNCH_TRAIN_F32(NQ_)                                                                                          \
-    hipLaunchKernelGGL(k_train_f32_dpp<NQ_>, dim3(ctx->Rpad / kWave, (ctx->N + 3) / 4), dim3(256), 0, ctx->stream,      \
+    hipLaunchKernelGGL(k_train_f32_dpp<NQ_>, dim3(rblocks, (ctx->N + per_block - 1) / per_block), dim3(64 * per_block), 0, ctx->stream, \
                        (const float *)ctx->d_somP, (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad,   \
                        ctx->d_key + (size_t)slot * ctx->N, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, prev)
     if (ctx->N <= 128) LAUNCH_TRAIN_F32(2); else LAUNCH_TRAIN_F32(4);
