@@ -47,8 +47,8 @@ MEASURED_VALU_LANE_OPS_T = 50.0     # subtract / fma stream, eight waves per SIM
 # by what the same counter reads for a device-to-device copy of known size; (bytes, the summary
 # under profiles/ that holds the readings).  Not measured in the run that prints the line.
 COUNTER_TRAFFIC_PER_IMAGE = {
-    ("cfg0", "distance"): (12.187e6 + 3.239e6, "profiles/cfg0_train_f32_counters.txt"),   # with the update of the image before
-    ("cfg0", "update"): ((18.466e6 + 0.774e6 + 1.712e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
+    ("cfg0", "distance"): (12.280e6 + 3.239e6, "profiles/cfg0_train_f32_counters.txt"),   # with the update of the image before
+    ("cfg0", "update"): ((28.149e6 + 0.774e6 + 1.711e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
     ("cfg1", "rotate"): ((95.405e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg1", "distance"): ((214.632e6 + 1.640e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg2", "distance"): (26.944e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
