@@ -712,16 +712,16 @@ struct PrevImage {
 };
 
 template <int NQ>     // neurons / 64, rounded up: keys and factors per lane in the search
-__global__ __launch_bounds__(384) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
+__global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                           unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
                                                           uint32_t R, uint32_t Rpad, PrevImage prev)
 {
     __shared__ v4f s_rot[2][64 * kDistRow / 4];
-    __shared__ float s_upd[6][2][64];          // per wave: the updated chunk on its way into the operand layout, two stages
+    __shared__ float s_upd[8][2][64];          // per wave: the updated chunk on its way into the operand layout, two stages
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t r0 = blockIdx.x * kWave;
-    // Four, five or six waves = neurons per block.  The first four move the rotation rows; a fifth and sixth only
+    // Four to eight waves = neurons per block.  The first four move the rotation rows; the others only
     // compute (where four neurons per block would make more blocks than the chip has CUs and fewer neurons per block
     // fewer, a CU with two blocks sets the pace for all: better every CU with one block and one or two SIMDs shared).
     const bool stages = wave < 4;
@@ -2232,11 +2232,12 @@ int run_train_f32(pink_hip_ctx *ctx, uint32_t slot, bool has_prev, uint32_t *bmu
         prev.bmu_out = bmu_prev;
         prev.counts = ctx->d_counts;
     }
-    // neurons (waves) per block: four, or the five or six that make the launch one block per CU where four do not
+    // neurons (waves) per block: four, or the five to eight that make the launch one block per CU where four do not
+    // (measured: 2 to 4 % per image; two blocks of five on a CU do not run side by side -- 28 against 21 us)
     const uint32_t rblocks = ctx->Rpad / kWave;
     uint32_t per_block = 4;
     if (rblocks * ((ctx->N + 3) / 4) > (uint32_t)ctx->num_cu)
-        for (uint32_t w = 5; w <= 6 && per_block == 4; ++w)
+        for (uint32_t w = 5; w <= 8 && per_block == 4; ++w)
             if (rblocks * ((ctx->N + w - 1) / w) <= (uint32_t)ctx->num_cu) per_block = w;
 #define LAUNCH_TRAIN_F32(NQ_)                                                                                          \
     hipLaunchKernelGGL(k_train_f32_dpp<NQ_>, dim3(rblocks, (ctx->N + per_block - 1) / per_block), dim3(64 * per_block), 0, ctx->stream, \

@@ -466,6 +466,8 @@ FUSED_TRAIN_SHAPES = [
     (257, 1, 14, 10, 8, False, 10, capi.QUADRATIC, capi.FLOAT, 3),    # ... and one more
     (103, 1, 20, 14, 360, True, 12, capi.QUADRATIC, capi.FLOAT, 3),   # 12 x 26 blocks of four neurons are more than the CUs: five per block, the last block three
     (110, 1, 20, 14, 360, True, 9, capi.CIRCULAR, capi.FLOAT, 3),     # ... six per block
+    (131, 1, 20, 14, 360, True, 9, capi.QUADRATIC, capi.FLOAT, 3),    # ... seven, three keys per lane in the search
+    (165, 1, 20, 14, 360, True, 12, capi.QUADRATIC, capi.FLOAT, 4),   # ... eight, the last block five
 ]
 
 
