@@ -2114,7 +2114,12 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
     // The 8 XCDs (each with its own L2) take rectangles of the tile grid: the split xr x xc = 8 with the fewest
     // operand rows per XCD (a tile row of variants and a tile column of neurons cost the same bytes).
-    const uint32_t row_tiles = ctx->Rp / 64, col_tiles = ctx->Np / 64;
+    // One image whose 32 x 32 tiles make no more blocks than there are CUs: a block per such tile over the whole k
+    // range, which finishes its tile itself (no partial sums in memory, no second kernel).
+    const uint32_t real32 = ((ctx->R + 31) / 32) * ((ctx->N + 31) / 32);
+    const bool tile32 = B == 1 && ctx->gslices > 1 && real32 <= (uint32_t)ctx->num_cu;
+    const uint32_t side = tile32 ? 32u : 64u;
+    const uint32_t row_tiles = ctx->Rp / side, col_tiles = ctx->Np / side;
     uint32_t xc = 1, cost = ~0u;
     for (uint32_t c = 1; c <= 8; c *= 2) {
         const uint32_t r = 8 / c, v = (row_tiles + r - 1) / r + (col_tiles + c - 1) / c;
@@ -2122,8 +2127,8 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     }
     const uint32_t rect_h = (row_tiles + 8 / xc - 1) / (8 / xc), rect_w = (col_tiles + xc - 1) / xc;
     const uint32_t tiles_per_xcd = rect_h * rect_w;
-    const uint32_t slices = B > 1 ? 1 : ctx->gslices;
-    const uint32_t ks_per = B > 1 ? (ctx->gKS + 3) / 4 : ctx->gks_per;
+    const uint32_t slices = B > 1 || tile32 ? 1 : ctx->gslices;
+    const uint32_t ks_per = B > 1 || tile32 ? (ctx->gKS + 3) / 4 : ctx->gks_per;
     GemmFinish fin{};
     long long *na = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, *na_other = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
     const long long *nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
@@ -2134,8 +2139,12 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
         // a block sees the whole k range: it finishes its tile itself
         fin.key = key; fin.na = na; fin.na_other = na_other; fin.N = ctx->N; fin.R = ctx->R;
     }
-    hipLaunchKernelGGL(k_dist_gemm_int<U16>, dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
-                       (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, slices, rect_h, rect_w, xc, fin);
+    if (tile32)
+        hipLaunchKernelGGL((k_dist_gemm_int<U16, 1>), dim3(8 * tiles_per_xcd, 1), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
+                           (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, 1u, rect_h, rect_w, xc, fin);
+    else
+        hipLaunchKernelGGL((k_dist_gemm_int<U16, 2>), dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
+                           (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, slices, rect_h, rect_w, xc, fin);
     if (slices == 1) return;
     const uint32_t rows_per_chunk = 32;
     hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
