@@ -1759,7 +1759,8 @@ struct pink_hip_ctx {
 
     // integer distances as an int8 MFMA GEMM with split k (training, SOMs of any size)
     bool gemm = false;
-    uint32_t gKS = 0, Np = 0, Rp = 0, gslices = 1, gks_per = 0;   // k-slices (blocks per tile), k-steps per wave
+    uint32_t gKS = 0, Np = 0, Rp = 0;
+    bool g_tile32 = false;     // one image: a block per 32 x 32 tile instead of 64 x 64 (few tiles, long rows)
     v4i *d_gPa = nullptr, *d_gPb = nullptr;
     v4i *d_gPa_alt = nullptr;             // small uint8 trainers: the SOM operand alternates between two buffers
     uint32_t pa_cur = 0;                   // ... which of them holds the current SOM
@@ -1768,7 +1769,6 @@ struct pink_hip_ctx {
     uint32_t *d_kbyte = nullptr;
     uint32_t *d_grow = nullptr, *d_gvariant = nullptr;   // variant index -> row of the variant operand, and back
     long long *d_gna = nullptr, *d_gnb = nullptr;
-    int *d_dot = nullptr;
 
     unsigned char *static_scratch = nullptr;   // this device's copy of the file-scope scratch array
 
@@ -2104,23 +2104,20 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 #undef LAUNCH_SG
 }
 
-// Distances of B images starting at image slot `slot`.  One image (training): k is cut into
-// ctx->gslices slices so that the chip is filled.  Several images (mapping): the images fill the
-// chip, every block takes the whole k range of its tile and finishes it, one launch for all.
+// Distances of B images starting at image slot `slot`: one launch, every block takes the whole k range of its
+// tile and finishes it.  Several images (mapping) fill the chip with 64 x 64 tiles; one image (training) with few
+// tiles and long rows takes 32 x 32 tiles (measured against 64 x 64 tiles with k cut across blocks and a second
+// kernel that adds the partial sums up, images/s of the whole training step: 253 tiles x 135 k-steps uint16 +17 %,
+// 299 x 64 uint16 +27 %, 414 x 64 uint16 +25 %, 299 x 128 uint8 +13 %, equal from 23 to 184 tiles).
 template <bool U16>
 void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
 {
     const uint32_t planes = U16 ? 2 : 1;
     const v4i *pb = ctx->d_gPb + (size_t)slot * planes * (ctx->Rp / 32) * ctx->gKS * 64;
+    const bool tile32 = B == 1 && ctx->g_tile32;
+    const uint32_t side = tile32 ? 32u : 64u;
     // The 8 XCDs (each with its own L2) take rectangles of the tile grid: the split xr x xc = 8 with the fewest
     // operand rows per XCD (a tile row of variants and a tile column of neurons cost the same bytes).
-    // One image that would otherwise be cut along k (few tiles of 64 x 64): a block per 32 x 32 tile over the whole k
-    // range, which finishes its tile itself -- no partial sums in memory, no second kernel (measured against the
-    // sliced form, images/s of the whole training step: 253 tiles x 135 k-steps uint16 +17 %, 299 x 64 uint16 +27 %,
-    // 414 x 64 uint16 +25 %, 299 x 128 uint8 +13 %, equal from 23 to 184 tiles).
-    const uint32_t real32 = ((ctx->R + 31) / 32) * ((ctx->N + 31) / 32);
-    const bool tile32 = B == 1 && ctx->gslices > 1 && real32 <= 2 * (uint32_t)ctx->num_cu;
-    const uint32_t side = tile32 ? 32u : 64u;
     const uint32_t row_tiles = ctx->Rp / side, col_tiles = ctx->Np / side;
     uint32_t xc = 1, cost = ~0u;
     for (uint32_t c = 1; c <= 8; c *= 2) {
@@ -2129,29 +2126,20 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     }
     const uint32_t rect_h = (row_tiles + 8 / xc - 1) / (8 / xc), rect_w = (col_tiles + xc - 1) / xc;
     const uint32_t tiles_per_xcd = rect_h * rect_w;
-    const uint32_t slices = B > 1 || tile32 ? 1 : ctx->gslices;
-    const uint32_t ks_per = B > 1 || tile32 ? (ctx->gKS + 3) / 4 : ctx->gks_per;
+    const uint32_t ks_per = (ctx->gKS + 3) / 4;
     GemmFinish fin{};
-    long long *na = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np, *na_other = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
-    const long long *nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
-    unsigned long long *key = ctx->d_key + (size_t)slot * ctx->N;
-    fin.nb = nb;
+    fin.key = ctx->d_key + (size_t)slot * ctx->N;
+    fin.na = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np;
+    fin.na_other = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
+    fin.nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
     fin.variant = ctx->d_gvariant;
-    if (slices == 1) {
-        // a block sees the whole k range: it finishes its tile itself
-        fin.key = key; fin.na = na; fin.na_other = na_other; fin.N = ctx->N; fin.R = ctx->R;
-    }
+    fin.N = ctx->N; fin.R = ctx->R;
     if (tile32)
         hipLaunchKernelGGL((k_dist_gemm_int<U16, 1>), dim3(8 * tiles_per_xcd, 1), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
-                           (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, 1u, rect_h, rect_w, xc, fin);
+                           ctx->Np, ctx->Rp, ctx->gKS, ks_per, rect_h, rect_w, xc, fin);
     else
-        hipLaunchKernelGGL((k_dist_gemm_int<U16, 2>), dim3(8 * tiles_per_xcd * slices, B), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
-                           (void *)ctx->d_dot, ctx->Np, ctx->Rp, ctx->gKS, ks_per, slices, rect_h, rect_w, xc, fin);
-    if (slices == 1) return;
-    const uint32_t rows_per_chunk = 32;
-    hipLaunchKernelGGL(k_dist_finish_int<U16>, dim3((ctx->N + 31) / 32, (ctx->R + rows_per_chunk - 1) / rows_per_chunk),
-                       dim3(256), 0, ctx->stream, (const void *)ctx->d_dot, na, na_other, nb, key, ctx->N, ctx->Np, ctx->R,
-                       ctx->Rp, ctx->gslices, rows_per_chunk, ctx->d_gvariant);
+        hipLaunchKernelGGL((k_dist_gemm_int<U16, 2>), dim3(8 * tiles_per_xcd, B), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
+                           ctx->Np, ctx->Rp, ctx->gKS, ks_per, rect_h, rect_w, xc, fin);
 }
 
 // Distances of B images starting at image slot `slot` on the matrix cores, float32.
@@ -2338,7 +2326,7 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_factors_t, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_somP_alt, ctx->d_bmu_group, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_dot, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
@@ -2552,7 +2540,7 @@ int init_ctx(pink_hip_ctx *ctx)
         HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ctx->lds_max));
     }
 
-    // Integer distances as a split-k int8 GEMM: all that is left of the integer modes.  Small
+    // Integer distances as an int8 GEMM: all that is left of the integer modes.  Small
     // problems pad their rows to one 64 x 64 tile; they are latency bound either way and the four
     // waves of a block still cut k four ways.
     {
@@ -2571,16 +2559,10 @@ int init_ctx(pink_hip_ctx *ctx)
             ctx->Np = round_up(ctx->N, 64);
             ctx->Rp = round_up(ctx->R, 64);
             const uint32_t tiles = (ctx->Np / 64) * (ctx->Rp / 64);
-            // k is cut into slices (blocks per tile, four waves each) so that a wave has about 16 k-steps
-            // (uint8: 64 MFMAs) or 11 (uint16: 176), never more blocks than CUs.  Cutting costs a second
-            // launch that adds the slices up; one slice finishes its tile itself.  Measured optima, images/s
-            // against one slice: 12 tiles x 235 k-steps uint8: 4 slices, +21 %; 24 x 254 uint8: 4, +15 %;
-            // 24 x 254 uint16: 6, +37 %; 72 x 135 uint16: 3; 24 x 64 uint8 and 84 x 141 uint8: 1.
+            // A launch of one image takes 32 x 32 tiles where 64 x 64 tiles would leave a wave more than about 16
+            // k-steps (uint8: 64 MFMAs) or 11 (uint16: 176) while at least half of the CUs stay without a block.
             const uint32_t per_wave = c.ed_type == PINK_HIP_UINT16 ? 11u : 16u;
-            uint32_t slices = (ctx->gKS + 4 * per_wave - 1) / (4 * per_wave);
-            slices = std::max(1u, std::min(slices, (uint32_t)ctx->num_cu / tiles));
-            ctx->gks_per = (ctx->gKS + 4 * slices - 1) / (4 * slices);
-            ctx->gslices = (ctx->gKS + 4 * ctx->gks_per - 1) / (4 * ctx->gks_per);
+            ctx->g_tile32 = ctx->gKS > 4 * per_wave && 2 * tiles <= (uint32_t)ctx->num_cu;
         }
     }
 
@@ -2693,7 +2675,6 @@ int init_ctx(pink_hip_ctx *ctx)
     } else if (ctx->gemm) {
         const size_t planes = c.ed_type == PINK_HIP_UINT16 ? 2 : 1;
         const size_t a_vec = planes * (ctx->Np / 32) * ctx->gKS * 64, b_vec = planes * (ctx->Rp / 32) * ctx->gKS * 64;
-        const size_t dot_n = ctx->gslices * planes * (size_t)ctx->Rp * ctx->Np;   // int32 (uint8) or int64 (uint16) per element
         TRY(dev_alloc(ctx, &ctx->d_gPa, a_vec));
         TRY(dev_alloc(ctx, &ctx->d_gPb, B * b_vec));
         TRY(dev_alloc(ctx, &ctx->d_gna, (size_t)2 * ctx->Np));   // two halves, see na_cur
@@ -2715,11 +2696,9 @@ int init_ctx(pink_hip_ctx *ctx)
             HIP_TRY(ctx, hipMemcpy(ctx->d_grow, row_of.data(), row_of.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
             HIP_TRY(ctx, hipMemcpy(ctx->d_gvariant, variant_of.data(), variant_of.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
         }
-        TRY(dev_alloc(ctx, &ctx->d_dot, dot_n));
         // rows beyond N / R and elements beyond the region are never written: they must read as zero
         HIP_TRY(ctx, hipMemset(ctx->d_gPa, 0, a_vec * sizeof(v4i)));
         HIP_TRY(ctx, hipMemset(ctx->d_gPb, 0, B * b_vec * sizeof(v4i)));
-        HIP_TRY(ctx, hipMemset(ctx->d_dot, 0, dot_n * sizeof(int)));
     } else if (ctx->mfma) {
         TRY(dev_alloc(ctx, &ctx->d_Pa, (size_t)ctx->NT * ctx->KS * 1024));
         TRY(dev_alloc(ctx, &ctx->d_na, (size_t)ctx->NT * 32));
@@ -3334,8 +3313,8 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
     // the kernels take the scratch where they take the context's own buffers in pink_hip_map_device
     struct Saved {
         unsigned long long *key; signed char *Pb; int *nb; v4i *gPb; long long *gnb; float *rot; void *rotT;
-        uint32_t Bcap, gslices, gks_per;
-    } const saved{ctx->d_key, ctx->d_Pb, ctx->d_nb, ctx->d_gPb, ctx->d_gnb, ctx->d_rot, ctx->d_rotT, ctx->Bcap, ctx->gslices, ctx->gks_per};
+        uint32_t Bcap;
+    } const saved{ctx->d_key, ctx->d_Pb, ctx->d_nb, ctx->d_gPb, ctx->d_gnb, ctx->d_rot, ctx->d_rotT, ctx->Bcap};
     unsigned char *at = ctx->static_scratch;
     auto carve = [&](size_t bytes_per_image) { unsigned char *p = at; at += (size_t)B * bytes_per_image; return p; };
     ctx->d_key = (unsigned long long *)carve(pc.key);
@@ -3346,12 +3325,6 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
     if (pc.rot) ctx->d_rot = (float *)carve(pc.rot);
     if (pc.rotT) ctx->d_rotT = carve(pc.rotT);
     ctx->Bcap = B;
-    if (ctx->gemm) {
-        // a block takes the whole k range of its tile also when a group holds a single image: no partial
-        // sums in memory (the context's own buffer for them is not used here)
-        ctx->gslices = 1;
-        ctx->gks_per = (ctx->gKS + 3) / 4;
-    }
     int rc = PINK_HIP_OK;
     for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += B) {
         const uint32_t b = std::min(B, n_images - done);
@@ -3361,7 +3334,7 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
                               dev_best_rot_out ? dev_best_rot_out + (size_t)done * ctx->N : nullptr, true);
     }
     ctx->d_key = saved.key; ctx->d_Pb = saved.Pb; ctx->d_nb = saved.nb; ctx->d_gPb = saved.gPb; ctx->d_gnb = saved.gnb;
-    ctx->d_rot = saved.rot; ctx->d_rotT = saved.rotT; ctx->Bcap = saved.Bcap; ctx->gslices = saved.gslices; ctx->gks_per = saved.gks_per;
+    ctx->d_rot = saved.rot; ctx->d_rotT = saved.rotT; ctx->Bcap = saved.Bcap;
     return rc;
 }
 
