@@ -51,8 +51,8 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg0", "update"): ((28.149e6 + 0.774e6 + 1.711e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
     ("cfg1", "rotate"): ((95.405e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg1", "distance"): ((214.632e6 + 1.640e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg2", "distance"): (26.944e6 + 7.078e6 + 5.927e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (27.029e6 + 20.734e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "distance"): (25.224e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (27.032e6 + 20.729e6, "profiles/cfg2_train_u16_counters.txt"),
     ("cfg3", "distance"): (874.783e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
     ("cfg3", "update"): (73.898e6 + 47.153e6 + (294.770e6 + 94.546e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
