@@ -452,6 +452,8 @@ FUSED_TRAIN_SHAPES = [
     (2, 1, 100, 257, 4, False, 257, capi.QUADRATIC, capi.UINT8, 2),   # 66 049: beyond the matrix-core path's row length
     (2, 1, 100, 256, 4, False, 256, capi.QUADRATIC, capi.UINT16, 2),  # 65 536 (uint16 sums reach 2^48 just above that)
     (12, 1, 64, 44, 360, True, 32, capi.QUADRATIC, capi.UINT16, 2),   # 720 variants, uint16 planes out of the rotation kernel
+    (70, 1, 40, 48, 36, True, 44, capi.QUADRATIC, capi.UINT16, 3),    # long rows, few tiles: 32 x 32 tiles (3 x 3 real ones among 16), each finished by its block
+    (70, 1, 40, 52, 36, True, 48, capi.QUADRATIC, capi.UINT8, 3),     # the same for uint8 (72 k-steps)
     # small uint8 trainers: distance, best match and update of an image in one launch
     (33, 1, 44, 40, 4, True, 40, capi.QUADRATIC, capi.UINT8, 5),      # 1600 elements per neuron, 50 k-steps (two batches of operand loads), a second column tile of one neuron
     (64, 1, 30, 28, 16, True, 20, capi.CIRCULAR, capi.UINT8, 5),      # 32 variants (a full row tile), eight stored variants staged in LDS
