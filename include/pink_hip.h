@@ -68,7 +68,7 @@ typedef enum {
     PINK_HIP_KERNEL_VALU = 1,      /* integer modes on the vector ALU in exact int32/int64                */
     PINK_HIP_KERNEL_MFMA = 2,      /* uint8 mapper, int8 MFMA, symmetries applied to the image variants   */
     PINK_HIP_KERNEL_MFMA_SYM = 3,  /* uint8 mapper, int8 MFMA, symmetries applied to the SOM once         */
-    PINK_HIP_KERNEL_MFMA_GEMM = 4, /* integer modes, trainer or mapper: split-k int8 MFMA GEMM (uint16 as 4 byte-plane products) */
+    PINK_HIP_KERNEL_MFMA_GEMM = 4, /* integer modes, trainer or mapper: int8 MFMA GEMM, one launch (uint16 as 4 byte-plane products) */
     PINK_HIP_KERNEL_MFMA_F32 = 5   /* float32, trainer or mapper, on request only: |a|^2 + |b|^2 - 2 a.b with float32 MFMA dot
                                       products -- not the CPU's summation order: distances agree to a relative tolerance, best
                                       rotations where candidates are not that close, trained weights drift */
