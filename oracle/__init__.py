@@ -161,6 +161,30 @@ def distance_matrix(s, som, rotated):
     return d, ssd, best
 
 
+def distance_matrix_pairwise(s, som, rotated):
+    """The same matrix with one functor call per pair (what distance_matrix is checked against)."""
+    som = np.ascontiguousarray(som, np.float32)
+    rotated = np.ascontiguousarray(rotated, np.float32)
+    d = np.empty(s.som_size, np.float32)
+    ssd = np.zeros(s.som_size, np.int64)
+    best = np.zeros(s.som_size, np.uint32)
+    lib().pink_oracle_distance_matrix_pairwise(C.byref(s), _p(som, C.c_float), _p(rotated, C.c_float),
+                                               _p(d, C.c_float), _p(ssd, C.c_int64), _p(best, C.c_uint32))
+    return d, ssd, best
+
+
+def distance_matrix_reference_loop(s, som, rotated):
+    """Float mode with the reference's own OpenMP structure (a parallel loop over rotations per neuron,
+    a call through a pointer and a critical section per pair)."""
+    som = np.ascontiguousarray(som, np.float32)
+    rotated = np.ascontiguousarray(rotated, np.float32)
+    d = np.empty(s.som_size, np.float32)
+    best = np.zeros(s.som_size, np.uint32)
+    lib().pink_oracle_distance_matrix_reference_loop(C.byref(s), _p(som, C.c_float), _p(rotated, C.c_float),
+                                                     _p(d, C.c_float), _p(best, C.c_uint32))
+    return d, best
+
+
 def update_factors(layout, dims, functor, sigma, damping, max_update_distance=-1.0):
     dims = np.asarray(dims, np.uint32)
     N = int(lib().pink_oracle_hex_size(C.c_uint32(int(dims[0])))) if layout == HEXAGONAL else int(np.prod(dims))

@@ -266,9 +266,11 @@ int32_t pink_oracle_quantise(float x, uint32_t ed_type)
  * d[n] starts at rotation 0, later rotations replace it only when strictly
  * smaller, so the first index attaining the minimum wins.  The OpenMP split
  * here keeps a per-thread (min, lowest index) and merges by (value, index), which
- * gives the one-thread answer for any thread count. */
-void pink_oracle_distance_matrix(const pink_oracle_shape *s, const float *som, const float *rotated,
-                                 float *dist_f32, int64_t *ssd_int, uint32_t *best_rot)
+ * gives the one-thread answer for any thread count.  One functor call per pair,
+ * as the reference makes them; pink_oracle_distance_matrix below gives the same
+ * bits faster and is checked against this form (tests/test_oracle_golden.py). */
+void pink_oracle_distance_matrix_pairwise(const pink_oracle_shape *s, const float *som, const float *rotated,
+                                          float *dist_f32, int64_t *ssd_int, uint32_t *best_rot)
 {
     const uint32_t N = s->som_size;
     const uint32_t R = s->num_rot * (s->use_flip ? 2 : 1);
@@ -326,6 +328,169 @@ void pink_oracle_distance_matrix(const pink_oracle_shape *s, const float *som, c
         free(qr);
     }
     free(off);
+}
+
+/* The same matrix with the reference's own parallel structure
+ * (generate_euclidean_distance_matrix.h:45-56): every neuron opens one `omp parallel for` over the
+ * rotations, every pair is one call through a function object (here a function pointer) and one
+ * `omp critical` section that compares and stores.  Like the reference with more than one thread,
+ * equal distances go to whichever thread enters first; what the benchmark's CPU baseline times.
+ * Float mode only (the reference's CPU path has no other). */
+typedef float (*pair_functor)(const float *, const float *, const uint32_t *, uint32_t);
+
+void pink_oracle_distance_matrix_reference_loop(const pink_oracle_shape *s, const float *som,
+                                                const float *rotated, float *dist_f32, uint32_t *best_rot)
+{
+    const uint32_t N = s->som_size;
+    const uint32_t R = s->num_rot * (s->use_flip ? 2 : 1);
+    const size_t nsz = (size_t)s->channels * s->neuron_dim * s->neuron_dim;
+    uint32_t E = pink_oracle_region(s->channels, s->neuron_dim, s->ed_dim, s->ed_shape, NULL);
+    uint32_t *off = (uint32_t *)malloc((size_t)(E ? E : 1) * sizeof(uint32_t));
+    pink_oracle_region(s->channels, s->neuron_dim, s->ed_dim, s->ed_shape, off);
+    volatile pair_functor functor = ssd_f32_offsets;
+
+    for (uint32_t n = 0; n < N; ++n) {
+        dist_f32[n] = functor(som + n * nsz, rotated, off, E);
+        best_rot[n] = 0;
+        #pragma omp parallel for
+        for (uint32_t r = 1; r < R; ++r) {
+            float t = functor(som + n * nsz, rotated + r * nsz, off, E);
+            #pragma omp critical
+            if (t < dist_f32[n]) { dist_f32[n] = t; best_rot[n] = r; }
+        }
+    }
+    free(off);
+}
+
+/* Sixteen rotations side by side.  Every pair still runs the functor's own sequence of operations in
+ * the functor's element order (float difference; square and sum in double; the sum rounded to float
+ * after every element); only which pairs share a vector instruction changes, so the results are the
+ * bits of ssd_f32_offsets / ssd_int_offsets.  rt = the region of the variants, element-major
+ * (rt[k * ld + r]). */
+#define PO_LANES 16
+typedef float   po_f4 __attribute__((vector_size(16)));
+typedef int32_t po_i4 __attribute__((vector_size(16)));
+typedef double  po_d4 __attribute__((vector_size(32)));
+
+__attribute__((target_clones("avx2", "default")))
+static void ssd_f32_lanes(const float *a, const float *rt0, const float *rt1, uint32_t n, float *out0, float *out1)
+{
+    /* two blocks of sixteen variants (eight independent chains of four lanes: a chain's step is a
+     * convert, an add and a convert back, a dozen cycles that the other chains fill) */
+    po_f4 ed0 = {0}, ed1 = {0}, ed2 = {0}, ed3 = {0}, ed4 = {0}, ed5 = {0}, ed6 = {0}, ed7 = {0};
+#define PO_STEP(ed, row, j) { po_f4 b; memcpy(&b, row + 4 * (j), sizeof b); po_f4 diff = av - b;         \
+                         po_d4 wide = __builtin_convertvector(diff, po_d4);                            \
+                         po_d4 sum = __builtin_convertvector(ed, po_d4) + wide * wide;                 \
+                         ed = __builtin_convertvector(sum, po_f4); }
+    for (uint32_t k = 0; k < n; ++k) {
+        const float *r0 = rt0 + (size_t)k * PO_LANES, *r1 = rt1 + (size_t)k * PO_LANES;
+        const po_f4 av = {a[k], a[k], a[k], a[k]};
+        PO_STEP(ed0, r0, 0) PO_STEP(ed1, r0, 1) PO_STEP(ed2, r0, 2) PO_STEP(ed3, r0, 3)
+        PO_STEP(ed4, r1, 0) PO_STEP(ed5, r1, 1) PO_STEP(ed6, r1, 2) PO_STEP(ed7, r1, 3)
+    }
+#undef PO_STEP
+    memcpy(out1, &ed4, 16); memcpy(out1 + 4, &ed5, 16); memcpy(out1 + 8, &ed6, 16); memcpy(out1 + 12, &ed7, 16);
+    memcpy(out0, &ed0, 16); memcpy(out0 + 4, &ed1, 16); memcpy(out0 + 8, &ed2, 16); memcpy(out0 + 12, &ed3, 16);
+}
+
+/* Integer pairs: double(ed) + double(diff)^2 is exact while every partial sum stays below 2^53
+ * (the functor's own condition), so the sum stays in double until the end. */
+__attribute__((target_clones("avx2", "default")))
+static void ssd_int_lanes(const int32_t *a, const int32_t *rt, uint32_t n, int64_t *out)
+{
+    po_d4 ed[4] = {{0}, {0}, {0}, {0}};
+    po_d4 ed0 = {0}, ed1 = {0}, ed2 = {0}, ed3 = {0};
+#define PO_STEP(ed, j) { po_i4 b; memcpy(&b, row + 4 * (j), sizeof b); po_i4 diff = av - b;              \
+                         po_d4 wide = __builtin_convertvector(diff, po_d4); ed = ed + wide * wide; }
+    for (uint32_t k = 0; k < n; ++k) {
+        const int32_t *row = rt + (size_t)k * PO_LANES;
+        const po_i4 av = {a[k], a[k], a[k], a[k]};
+        PO_STEP(ed0, 0) PO_STEP(ed1, 1) PO_STEP(ed2, 2) PO_STEP(ed3, 3)
+    }
+#undef PO_STEP
+    ed[0] = ed0; ed[1] = ed1; ed[2] = ed2; ed[3] = ed3;
+    for (int j = 0; j < PO_LANES; ++j) out[j] = (int64_t)ed[j / 4][j % 4];
+}
+
+/* generate_euclidean_distance_matrix.h:19-59, the answer of its one-thread run (first rotation
+ * attaining the minimum), evaluated sixteen rotations at a time.  Bit-identical to
+ * pink_oracle_distance_matrix_pairwise. */
+void pink_oracle_distance_matrix(const pink_oracle_shape *s, const float *som, const float *rotated,
+                                 float *dist_f32, int64_t *ssd_int, uint32_t *best_rot)
+{
+    const uint32_t N = s->som_size;
+    const uint32_t R = s->num_rot * (s->use_flip ? 2 : 1);
+    const size_t nsz = (size_t)s->channels * s->neuron_dim * s->neuron_dim;
+    const uint32_t blocks = (R + PO_LANES - 1) / PO_LANES;
+    const size_t ld = (size_t)blocks * PO_LANES;
+    uint32_t E = pink_oracle_region(s->channels, s->neuron_dim, s->ed_dim, s->ed_shape, NULL);
+    const size_t Ea = E ? E : 1;
+    uint32_t *off = (uint32_t *)malloc(Ea * sizeof(uint32_t));
+    pink_oracle_region(s->channels, s->neuron_dim, s->ed_dim, s->ed_shape, off);
+    const int is_float = s->ed_type == PINK_ORACLE_FLOAT;
+    const uint32_t factor = pink_oracle_quant_factor(s->ed_type);
+    /* the region of the variants, sixteen variants at a time and element-major inside such a block
+     * (rt[(block * E + k) * 16 + lane]), and the region of every neuron, gathered; 4-byte elements:
+     * floats, or the quantised integers of the integer modes.  all[n * ld + r] = the pair's sum. */
+    uint32_t *rt = (uint32_t *)calloc(Ea * ld, 4);
+    uint32_t *sr = (uint32_t *)malloc((size_t)N * Ea * 4);
+    int64_t *all = (int64_t *)malloc((size_t)N * ld * sizeof(int64_t));
+
+    #pragma omp parallel
+    {
+        #pragma omp for schedule(static) nowait
+        for (uint32_t r = 0; r < R; ++r)
+            for (uint32_t k = 0; k < E; ++k) {
+                float v = rotated[r * nsz + off[k]];
+                uint32_t *dst = &rt[((size_t)(r / PO_LANES) * E + k) * PO_LANES + r % PO_LANES];
+                if (is_float) memcpy(dst, &v, 4);
+                else *dst = (uint32_t)pink_oracle_quantise(v, s->ed_type);
+            }
+        #pragma omp for schedule(static)
+        for (uint32_t n = 0; n < N; ++n)
+            for (uint32_t k = 0; k < E; ++k) {
+                float v = som[n * nsz + off[k]];
+                if (is_float) memcpy(&sr[(size_t)n * E + k], &v, 4);
+                else sr[(size_t)n * E + k] = (uint32_t)pink_oracle_quantise(v, s->ed_type);
+            }
+        /* float: two blocks per call (an odd last block runs beside itself) */
+        #pragma omp for schedule(dynamic, 1)
+        for (uint32_t blk = 0; blk < blocks; blk += is_float ? 2 : 1) {
+            const uint32_t blk1 = blk + 1 < blocks ? blk + 1 : blk;
+            for (uint32_t n = 0; n < N; ++n) {
+                int64_t *out = all + (size_t)n * ld + (size_t)blk * PO_LANES;
+                int64_t *out1 = all + (size_t)n * ld + (size_t)blk1 * PO_LANES;
+                if (is_float) ssd_f32_lanes((const float *)sr + (size_t)n * E,
+                                            (const float *)rt + (size_t)blk * E * PO_LANES,
+                                            (const float *)rt + (size_t)blk1 * E * PO_LANES, E,
+                                            (float *)out, (float *)out1);
+                else ssd_int_lanes((const int32_t *)sr + (size_t)n * E,
+                                   (const int32_t *)rt + (size_t)blk * E * PO_LANES, E, out);
+            }
+        }
+        #pragma omp for schedule(static)
+        for (uint32_t n = 0; n < N; ++n) {
+            uint32_t bmin = 0;
+            if (is_float) {
+                float fmin = 0.0f;
+                for (uint32_t r = 0; r < R; ++r) {
+                    const float t = ((const float *)(all + (size_t)n * ld + (size_t)(r / PO_LANES) * PO_LANES))[r % PO_LANES];
+                    if (r == 0 || t < fmin) { fmin = t; bmin = r; }
+                }
+                dist_f32[n] = fmin;
+            } else {
+                int64_t imin = 0;
+                for (uint32_t r = 0; r < R; ++r) {
+                    const int64_t t = all[(size_t)n * ld + r];
+                    if (r == 0 || t < imin) { imin = t; bmin = r; }
+                }
+                if (ssd_int) ssd_int[n] = imin;
+                dist_f32[n] = (float)((double)imin / ((double)factor * (double)factor));
+            }
+            best_rot[n] = bmin;
+        }
+    }
+    free(rt); free(sr); free(all); free(off);
 }
 
 /* ------------------------------------------------------------------------ */

@@ -94,6 +94,16 @@ uint32_t pink_oracle_quant_factor(uint32_t ed_type);
  * exact integer SSD and dist_f32 = float(double(ssd) / double(factor^2)). */
 void pink_oracle_distance_matrix(const pink_oracle_shape *s, const float *som, const float *rotated,
                                  float *dist_f32, int64_t *ssd_int, uint32_t *best_rot);
+/* The same matrix, one functor call per pair as the reference makes them (the definition the
+ * sixteen-rotations-at-a-time form above is checked against, bit for bit). */
+void pink_oracle_distance_matrix_pairwise(const pink_oracle_shape *s, const float *som, const float *rotated,
+                                          float *dist_f32, int64_t *ssd_int, uint32_t *best_rot);
+/* Float mode with the reference's own parallel structure (generate_euclidean_distance_matrix.h:45-56):
+ * `omp parallel for` over the rotations of one neuron, one call through a function pointer and one
+ * `omp critical` section per pair.  With several threads equal distances go to the thread that enters
+ * first, as in the reference.  What the benchmark's CPU baseline times. */
+void pink_oracle_distance_matrix_reference_loop(const pink_oracle_shape *s, const float *som,
+                                                const float *rotated, float *dist_f32, uint32_t *best_rot);
 
 /* ---- SOM-grid distances, neighbourhood functors, update factors ----------- */
 uint32_t pink_oracle_hex_size(uint32_t dim);

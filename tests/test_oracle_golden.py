@@ -263,3 +263,53 @@ def test_variant_invariants():
         assert np.array_equal(out[k + nrr], np.rot90(out[k], k=-1, axes=(1, 2)))
     for k in range(nrot):
         assert np.array_equal(out[k + nrot], out[k][:, ::-1, :])
+
+
+@pytest.mark.parametrize("ed_type", [O.FLOAT, O.UINT8, O.UINT16])
+@pytest.mark.parametrize("N,C,I,D,e,shape_,nrot,flip", [
+    (7, 1, 20, 14, 9, O.QUADRATIC, 12, True),       # 24 variants: one full block of 16 and half a block
+    (5, 3, 12, 9, 6, O.QUADRATIC, 36, True),        # 72 variants: an odd number of blocks
+    (9, 1, 24, 17, 11, O.CIRCULAR, 8, False),       # 8 variants: less than one block; odd diameter
+    (4, 1, 10, 10, 10, O.QUADRATIC, 4, True),       # permutations only
+    (3, 2, 16, 12, 8, O.CIRCULAR, 20, True),        # 3-D circular: channel 0 counted twice
+])
+def test_distance_matrix_forms_agree_bit_for_bit(ed_type, N, C, I, D, e, shape_, nrot, flip):
+    """The sixteen-variants-at-a-time evaluation against the definition: one functor call per pair."""
+    rng = np.random.default_rng(1000 * ed_type + N)
+    R = nrot * (2 if flip else 1)
+    s = O.shape(N, C, I, D, nrot, flip, e, shape_, ed_type)
+    for trial in range(3):
+        som = rng.random((N, C * D * D), dtype=np.float32)
+        img = rng.random(C * I * I, dtype=np.float32)
+        if trial == 1:                                  # few levels: equal distances between variants
+            som = np.round(som * 3) / np.float32(3)
+            img = np.round(img * 2) / np.float32(2)
+        if trial == 2:                                  # a neuron that is a variant: distance 0 late in the list
+            som[N - 1] = O.rotated_images(img, C, I, D, nrot, flip).reshape(R, -1)[R - 1]
+        rot = O.rotated_images(img, C, I, D, nrot, flip).reshape(R, -1)
+        d0, ssd0, best0 = O.distance_matrix_pairwise(s, som, rot)
+        d1, ssd1, best1 = O.distance_matrix(s, som, rot)
+        assert np.array_equal(d0.view(np.uint32), d1.view(np.uint32))
+        assert np.array_equal(ssd0, ssd1)
+        assert np.array_equal(best0, best1)
+
+
+def test_distance_matrix_reference_loop_one_thread():
+    """The reference's own loop structure gives the one-thread answer when run on one thread (with more,
+    equal distances go to whichever thread comes first, as in the reference)."""
+    rng = np.random.default_rng(5)
+    N, C, I, D, e, nrot = 6, 1, 20, 14, 9, 24
+    s = O.shape(N, C, I, D, nrot, True, e)
+    som = rng.random((N, C * D * D), dtype=np.float32)
+    rot = O.rotated_images(rng.random(C * I * I, dtype=np.float32), C, I, D, nrot, True).reshape(2 * nrot, -1)
+    d0, _, best0 = O.distance_matrix_pairwise(s, som, rot)
+    before = O.num_threads()
+    O.set_num_threads(1)
+    try:
+        d1, best1 = O.distance_matrix_reference_loop(s, som, rot)
+    finally:
+        O.set_num_threads(before)
+    assert np.array_equal(d0.view(np.uint32), d1.view(np.uint32))
+    assert np.array_equal(best0, best1)
+    d2, best2 = O.distance_matrix_reference_loop(s, som, rot)     # all threads: same distances
+    assert np.array_equal(d0.view(np.uint32), d2.view(np.uint32))
