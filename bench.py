@@ -102,10 +102,30 @@ def algorithmic_per_image(w, E, path):
     }
 
 
+def distance_path_name(w, path, times):
+    """The kernel that computed the distances in this run, by the library's path and what was launched."""
+    from pink_amd import capi
+    if w.ed_type == capi.FLOAT and path != capi.KERNEL_MFMA_F32:
+        if w.mode == "train" and 0 < times["update"][0] < times["distance"][0]:
+            return "float32 vector ALU, one (neuron, variant) pair per lane, DPP broadcast; the launch also applies the update of the image before"
+        return "float32 vector ALU, one (neuron, variant) pair per lane"
+    if w.mode == "train" and path == capi.KERNEL_MFMA_GEMM and times["distance"][0] == 0:
+        return "int8 MFMA inside the one launch per image of a small uint8 trainer (distances, best match, update)"
+    return {capi.KERNEL_VALU: "integer vector ALU", capi.KERNEL_MFMA: "int8 MFMA, image-side symmetries, SOM operand in LDS",
+            capi.KERNEL_MFMA_SYM: "int8 MFMA, SOM-side symmetries, SOM operand in registers",
+            capi.KERNEL_MFMA_GEMM: "int8 MFMA GEMM, one launch, 64x64 or 32x32 tiles over the whole k range, finished by their blocks",
+            capi.KERNEL_MFMA_F32: "float32 MFMA GEMM (recast, on request)"}[path]
+
+
 def cpu_baseline(w, som0, imgs_host, budget_s, quick=False):
-    """The CPU oracle on a bounded sample of the workload: all host threads, one thread, and, for the
-    integer workloads, the float32 arithmetic that the reference's own CPU path would run on them
-    (it has no integer mode)."""
+    """The CPU path on a bounded sample of the workload, on this host's cores.
+
+    `value`: the oracle run with the reference's own parallel structure
+    (generate_euclidean_distance_matrix.h:45-56: per neuron an `omp parallel for` over the rotations, one call
+    through a function pointer and one `omp critical` section per pair) in float32, the arithmetic the
+    reference's CPU path uses whatever the distance type (it has no integer mode).  `port`: the oracle's own,
+    leaner evaluation (sixteen variants side by side in vector registers, neurons and variant blocks spread
+    over the threads) in the workload's distance type: the faster CPU figure, not what the reference runs."""
     import oracle as O
     from pink_amd import capi, synthetic
     F = synthetic.update_factors(w) if w.mode == "train" else None
@@ -123,31 +143,35 @@ def cpu_baseline(w, som0, imgs_host, budget_s, quick=False):
             O.train(s, som0.copy(), imgs_host[:n], F)
         return time.perf_counter() - t
 
-    def rate(s, nthreads, budget):
+    def rate(s, form, nthreads, budget):
+        O.set_distance_form(form)
         O.set_num_threads(nthreads)
-        n_all = len(imgs_host)
-        run(s, min(2, n_all))                          # warm-up
-        probe_n = min(4 if nthreads > 1 else 1, n_all)
-        probe = run(s, probe_n)
-        n = int(max(probe_n, min(n_all, budget / max(probe / probe_n, 1e-6))))
-        dt = run(s, n)
-        O.set_num_threads(threads)
+        try:
+            n_all = len(imgs_host)
+            probe = run(s, 1)                              # warm-up, and how long an image takes
+            n, dt = 1, probe
+            if probe < budget / 2:
+                n = int(max(1, min(n_all, budget / max(probe, 1e-6))))
+                dt = run(s, n)
+        finally:
+            O.set_num_threads(threads)
+            O.set_distance_form(O.LANES)
         return n / dt, n, dt
 
-    v, n, dt = rate(shape(w.ed_type), threads, budget_s)
+    v, n, dt = rate(shape(capi.FLOAT), O.REFERENCE_LOOP, threads, budget_s)
     out = {"value": round(v, 3), "unit": "images/s", "cores": threads, "kind": "port",
-           "sample": "%d images of %s, %.1f s, OpenMP over rotations" % (n, w.name, dt),
-           "note": "the port keeps the reference's arithmetic and loop order but its parallel loop is leaner than the "
-                   "reference's (one critical section per thread, no std::function call per pair: "
-                   "generate_euclidean_distance_matrix.h:45-56), so it is somewhat faster than the reference's CPU path"}
+           "sample": "%d images of %s, %.1f s" % (n, w.name, dt),
+           "structure": "the oracle with the reference's own loop (generate_euclidean_distance_matrix.h:45-56): omp parallel "
+                        "for over the rotations of one neuron, a call through a function pointer and an omp critical section "
+                        "per pair; float32, the arithmetic of the reference's CPU path whatever the distance type"}
+    vp, np_, dtp = rate(shape(w.ed_type), O.LANES, threads, budget_s / 3)
+    out["port"] = {"value": round(vp, 3), "cores": threads, "dtype": DTYPE_NAME[w.ed_type],
+                   "sample": "%d images, %.1f s" % (np_, dtp),
+                   "what": "the oracle's own evaluation in the workload's distance type: sixteen variants side by side in "
+                           "vector registers, threads over neurons and variant blocks; same results, leaner than the reference"}
     if not quick:
-        v1, n1, dt1 = rate(shape(w.ed_type), 1, budget_s / 3)
+        v1, n1, dt1 = rate(shape(capi.FLOAT), O.REFERENCE_LOOP, 1, budget_s / 3)
         out["one_thread"] = {"value": round(v1, 3), "sample": "%d images, %.1f s" % (n1, dt1)}
-    if w.ed_type != capi.FLOAT:
-        vf, nf, dtf = rate(shape(capi.FLOAT), threads, budget_s / 3)
-        out["float32_cpu_path"] = {"value": round(vf, 3), "cores": threads, "sample": "%d images, %.1f s" % (nf, dtf),
-                                   "what": "the same workload in float32: the arithmetic the reference's CPU path "
-                                           "uses whatever the distance type (it has no integer mode)"}
     return out
 
 
@@ -240,6 +264,7 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
     imgs_per_launch = prof_images / max(launches, 1)
     per_s = imgs_per_launch / (avg_ms * 1e-3)
     notes = None
+    second_peak = None
     if dominant == "distance" and path == capi.KERNEL_MFMA_F32:
         bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
@@ -247,8 +272,10 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
                  "order (distances to a relative tolerance only); never the default")
     elif dominant == "distance" and w.ed_type == capi.FLOAT:
         # direct float32 form on the vector ALU: subtract + fma per pair element, counted as 2 ops
-        bound, unit, peak = "mfma", "TFLOP/s", FP32_PEAK_TFLOPS
+        bound, unit, peak = "valu", "TFLOP/s", FP32_PEAK_TFLOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
+        second_peak = ("non-packed vector-ALU stream measured on this pool (subtract + fma, eight waves per SIMD)",
+                       MEASURED_VALU_LANE_OPS_T)
         notes = ("compute bound on the vector ALU: bit-faithful sequential fma per (neuron, rotation), one subtract + "
                  "one fma per pair element (counted as 2 operations); non-packed instructions (packed FP32 is disabled in "
                  "this build) issue at 3.15 clocks per wave at best, measured: %.0f T operations/s = about a third of the "
@@ -261,6 +288,7 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
     elif dominant == "distance" and path in (capi.KERNEL_MFMA_SYM, capi.KERNEL_MFMA_GEMM, capi.KERNEL_MFMA):
         bound, unit, peak = "mfma", "TOP/s", MFMA_INT8_PEAK_TOPS
         achieved = alg["distance"]["ops"] * per_s / 1e12
+        second_peak = ("int8 MFMA stream measured on this pool (all SIMDs issuing)", MEASURED_INT8_MFMA_TOPS)
         notes = "int8 MFMA; measured MFMA peak on this pool %.0f TOP/s" % MEASURED_INT8_MFMA_TOPS
         if w.ed_type == capi.UINT16:
             notes += "; uint16 runs four byte-plane products per pair element, counted once"
@@ -284,9 +312,11 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
         "share_of_kernel_time": round(ms / total_ms, 4),
         "kernel_ms": {k: round(v[1], 4) for k, v in times.items()},
         "kernel_us_per_image": {k: round(v[1] * 1e3 / prof_images, 4) for k, v in times.items()},
-        "distance_path": {1: "vector ALU", 2: "int8 MFMA, image-side symmetries", 3: "int8 MFMA, SOM-side symmetries",
-                          4: "int8 MFMA GEMM, split k", 5: "float32 MFMA GEMM, split k (recast, on request)"}[path],
+        "distance_path": distance_path_name(w, path, times),
     }
+    if second_peak:
+        roofline["measured_ceiling"] = {"what": second_peak[0], "peak": second_peak[1], "unit": unit,
+                                        "frac": round(achieved / second_peak[1], 5)}
     if traffic:
         roofline["traffic_source"] = traffic[1] + " (rocprofv3 counters of an earlier run of this command, not of this run)"
     if notes:
@@ -334,7 +364,7 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
     torch.cuda.empty_cache()
     return {
         "metric": ("map" if w.mode == "map" else "train") + " images/sec @%d rot x flip" % w.R,
-        "value": round(value, 2), "unit": "images/s", "steps": steps, "warmup": warmup,
+        "value": round(value, 2), "device_resident": round(value, 2), "unit": "images/s", "steps": steps, "warmup": warmup,
         "ms_per_step": round(elapsed / steps * 1e3, 4), "dtype": DTYPE_NAME[w.ed_type],
         "config": {"workload": w.name, "mode": w.mode, "images_per_step": n_images, "images_in_config": w.n_images,
                    "som_size": w.som_size, "neuron": [w.channels, w.neuron_dim, w.neuron_dim],
@@ -386,6 +416,9 @@ def main():
         "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic", "config": head["config"],
+        "value_is": "device_resident: images in HBM when the clock starts, the trainer's final SOM copied back inside it; "
+                    "host_inclusive.value is the same step through the host-pointer entry points (H2D and D2H inside the clock)",
+        "device_resident": head["value"],
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "host_inclusive": head["host_inclusive"],
         "setup_s": head["setup_s"],
     }
@@ -397,7 +430,7 @@ def main():
             wu, st = SIDE_STEPS[name]
             r = run_workload(name, st, wu, min(SIDE_IMAGES[name], synthetic.WORKLOADS[name].n_images), "auto",
                              0.0 if args.no_cpu_baseline else 5.0, not args.no_host_inclusive, True)
-            side[name] = {k: r[k] for k in ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "config",
+            side[name] = {k: r[k] for k in ("metric", "value", "device_resident", "unit", "steps", "warmup", "ms_per_step", "dtype", "config",
                                             "roofline", "cpu_baseline", "host_inclusive")}
         out["all_configs"] = side
     print(json.dumps(out))

@@ -252,6 +252,14 @@ def map_images(s, som, images):
     return heat, best
 
 
+LANES, PAIRWISE, REFERENCE_LOOP = 0, 1, 2
+
+
+def set_distance_form(form):
+    """Which evaluation of the distance matrix train() and map_images() use (LANES by default)."""
+    assert lib().pink_oracle_set_distance_form(C.c_int(form)) == 0
+
+
 def num_threads():
     return int(lib().pink_oracle_num_threads())
 

@@ -633,6 +633,33 @@ void pink_oracle_update(float *som, uint32_t som_size, uint32_t neuron_size, con
     }
 }
 
+/* Which evaluation of the distance matrix pink_oracle_train / pink_oracle_map use: 0 = sixteen variants at
+ * a time (default), 1 = one functor call per pair, 2 = the reference's own OpenMP structure (float mode
+ * only: the reference's CPU path has no other; what the benchmark's CPU baseline times).  All three give the
+ * same distances; with form 2 on several threads equal distances go to the thread that enters first. */
+static int g_distance_form = 0;
+
+int pink_oracle_set_distance_form(int form)
+{
+    if (form < 0 || form > 2) return -1;
+    g_distance_form = form;
+    return 0;
+}
+
+static int distance_matrix_by_form(const pink_oracle_shape *s, const float *som, const float *rotated,
+                                   float *dist_f32, int64_t *ssd_int, uint32_t *best_rot)
+{
+    if (g_distance_form == 2) {
+        if (s->ed_type != PINK_ORACLE_FLOAT) return -2;
+        pink_oracle_distance_matrix_reference_loop(s, som, rotated, dist_f32, best_rot);
+    } else if (g_distance_form == 1) {
+        pink_oracle_distance_matrix_pairwise(s, som, rotated, dist_f32, ssd_int, best_rot);
+    } else {
+        pink_oracle_distance_matrix(s, som, rotated, dist_f32, ssd_int, best_rot);
+    }
+    return 0;
+}
+
 /* SelfOrganizingMapLib/Trainer.h:133-186 */
 int pink_oracle_train_step(const pink_oracle_shape *s, float *som, const float *image,
                            const float *factors, float *scratch_rot, uint32_t *bmu_out,
@@ -649,7 +676,7 @@ int pink_oracle_train_step(const pink_oracle_shape *s, float *som, const float *
 
     pink_oracle_rotated_images(image, s->channels, s->image_dim, s->neuron_dim, s->num_rot,
                                (int)s->use_flip, rot);
-    pink_oracle_distance_matrix(s, som, rot, dist, ssd, best);
+    if (distance_matrix_by_form(s, som, rot, dist, ssd, best)) { if (!scratch_rot) free(rot); free(dist); free(ssd); free(best); return -2; }
     uint32_t bmu = pink_oracle_bmu(s, dist, ssd);
     pink_oracle_update(som, N, (uint32_t)nsz, rot, best, bmu, factors);
 
@@ -696,7 +723,7 @@ int pink_oracle_map(const pink_oracle_shape *s, const float *som, const float *i
                                    s->num_rot, (int)s->use_flip, rot);
         float *d = heatmap_out + (size_t)i * N;
         memset(best, 0, N * sizeof(uint32_t));
-        pink_oracle_distance_matrix(s, som, rot, d, NULL, best);
+        if (distance_matrix_by_form(s, som, rot, d, NULL, best)) { free(rot); free(best); return -2; }
         for (uint32_t n = 0; n < N; ++n) d[n] = sqrtf(d[n]);
         if (best_rot_out) memcpy(best_rot_out + (size_t)i * N, best, N * sizeof(uint32_t));
     }

@@ -105,6 +105,11 @@ void pink_oracle_distance_matrix_pairwise(const pink_oracle_shape *s, const floa
 void pink_oracle_distance_matrix_reference_loop(const pink_oracle_shape *s, const float *som,
                                                 const float *rotated, float *dist_f32, uint32_t *best_rot);
 
+/* Which of the three evaluations above pink_oracle_train / pink_oracle_map use: 0 = sixteen variants at a time
+ * (default), 1 = pairwise, 2 = the reference's loop structure (float mode only; -2 from train / map otherwise).
+ * Returns 0, or -1 for an unknown form.  Process-wide. */
+int pink_oracle_set_distance_form(int form);
+
 /* ---- SOM-grid distances, neighbourhood functors, update factors ----------- */
 uint32_t pink_oracle_hex_size(uint32_t dim);
 float pink_oracle_cartesian_distance(const uint32_t *dims, uint32_t ndims, uint32_t i1, uint32_t i2);

@@ -2,12 +2,16 @@
 free-running weights, as the reference's own comparison does (test/CudaTest/compare_trainer_cpu.cu:49-98,
 gate 1e-4 on the weights).  Every case also says whether the weights came out bit-equal.
 
-cfg0 (2 000 images, float32) and cfg4 (60 000 images, uint8) run their whole epoch; cfg2 (uint16,
-331 neurons of 106 x 106) and cfg3 (float32, 1 600 neurons of 3 x 70 x 70) run as many images as the
-oracle finishes in seconds, with launch groups small enough that several group boundaries are crossed.
+cfg0 (2 000 images, float32) and cfg4 (60 000 images, uint8) run their whole epoch beside the oracle; cfg2
+(uint16, 331 neurons of 106 x 106, 10 000 images) and cfg3 (float32, 1 600 neurons of 3 x 70 x 70, 5 000
+images) run theirs against what the oracle recorded when it trained the same epoch once
+(tests/golden/epoch_cfg2.npz, epoch_cfg3.npz), and a few dozen images beside the oracle with launch groups
+small enough that several group boundaries are crossed.
 The mapper is then checked on the SOM that the cfg0 epoch leaves: images whose pixels quantise to a few
 dozen levels against smooth neurons, where equal integer distances are common.
 """
+import hashlib
+import os
 import sys
 
 import numpy as np
@@ -83,6 +87,54 @@ def test_cfg3_float32_across_group_boundaries():
     assert diff <= 1e-4
     assert np.array_equal(bmu, obmu)
     assert equal
+
+
+def _sha(a):
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg3"])
+def test_whole_epoch_against_the_recorded_oracle_epoch(name):
+    """cfg2 (10 000 images, uint16) and cfg3 (5 000 images, float32, three channels): the whole epoch on the
+    device against what the CPU oracle left when it trained the same epoch once, where the fixture was made
+    (tests/golden/make_epoch_vectors.py -> tests/golden/epoch_<cfg>.npz; the oracle needs a quarter of an hour
+    to an hour for them).  Gate as compare_trainer_cpu.cu:76 (1e-4 on the weights, here on every 997th weight and on
+    the neurons' sums); asserted beyond it: every best match equal and the SHA-256 of the weights equal."""
+    w = synthetic.WORKLOADS[name]
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "epoch_%s.npz" % name))
+    n, piece = int(fx["n_images"]), int(fx["piece"])
+    assert n == w.n_images and str(fx["workload"]) == w.name
+    imgs = synthetic.images(w, n)
+    som0 = synthetic.initial_som(w)
+    F = synthetic.update_factors(w)
+    # the inputs are built on this host: other bits here (another libm, another numpy) are not the device's doing
+    assert _sha(imgs) == str(fx["images_sha256"]), "this host builds other synthetic images than the fixture's"
+    assert _sha(F) == str(fx["factors_sha256"]), "this host builds another update-factor matrix than the fixture's"
+    assert _sha(som0) == str(fx["som0_sha256"])
+    say("epoch", name, n, "images against the recorded oracle epoch")
+    first_departure = None
+    with synthetic.make_context(w) as ctx:
+        ctx.set_som(som0)
+        bmu = []
+        for k, i in enumerate(range(0, n, piece)):
+            bmu.append(ctx.train(imgs[i:i + piece]))
+            if first_departure is None and _sha(ctx.get_som()) != str(fx["checkpoints"][k]):
+                first_departure = i
+        bmu = np.concatenate(bmu)
+        got = ctx.get_som()
+        counts = ctx.update_counts()
+    flat = got.reshape(-1)
+    slice_diff = float(np.abs(flat[fx["slice_index"]] - fx["slice_values"]).max())
+    sums = got.astype(np.float64).sum(1)
+    sum_diff = float(np.abs(sums - fx["neuron_sums"]).max() / w.neuron_size)
+    agree = float((bmu == fx["bmu"]).mean())
+    equal = _sha(got) == str(fx["som_sha256"])
+    say("   best-match agreement %.6f, max difference on the weight slice %.3g, mean per neuron %.3g, bit-equal: %s, "
+        "first piece that departs: %s" % (agree, slice_diff, sum_diff, equal, first_departure))
+    assert slice_diff <= 1e-4 and sum_diff <= 1e-4           # the gate
+    assert np.array_equal(bmu, fx["bmu"])
+    assert np.array_equal(counts, np.bincount(fx["bmu"], minlength=w.som_size))
+    assert equal and first_departure is None
 
 
 @pytest.fixture(scope="module")
