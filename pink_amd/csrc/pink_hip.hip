@@ -44,6 +44,24 @@
 // current device (the name below is a host-side stand-in, not a device address).
 static __device__ __align__(256) unsigned char scratch[PINK_HIP_STATIC_SCRATCH_BYTES];
 
+// Timestamp probes, in builds made with -DPINK_PROBE only (measurement builds; the shipped library has
+// none): wave w of block b of kernel k stores the 100 MHz constant clock at the places marked
+// PROBE(k, b, slot); pink_hip_probe_read copies the stamps of the last launch of each kernel out.
+#ifdef PINK_PROBE
+constexpr uint32_t kProbeKernels = 4, kProbeBlocks = 2048, kProbeWaves = 8, kProbeSlots = 8;
+static __device__ unsigned long long g_probe[kProbeKernels * kProbeBlocks * kProbeWaves * kProbeSlots];
+__device__ __forceinline__ void probe_stamp(uint32_t kernel, uint32_t block, uint32_t slot)
+{
+    if ((threadIdx.x & 63) == 0 && block < kProbeBlocks)
+        g_probe[((kernel * kProbeBlocks + block) * kProbeWaves + ((threadIdx.x >> 6) & (kProbeWaves - 1))) * kProbeSlots + slot] =
+            wall_clock64();
+}
+#define PROBE(kernel, block, slot) probe_stamp(kernel, block, slot)
+#else
+#define PROBE(kernel, block, slot) ((void)0)
+#endif
+constexpr uint32_t kProbeRotate = 0, kProbeGemm = 1, kProbeUpdate = 2, kProbeTrainF32 = 3;
+
 namespace {
 
 constexpr uint32_t kWave = 64;
@@ -177,6 +195,48 @@ __device__ __forceinline__ float base_pixel(const float *__restrict__ img, uint3
     return __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d);
 }
 
+// base_pixel for U pixels of a base rotation i > 0 at once, without branches: the 4 U image taps are all
+// requested before the first is used (a block's fill of its LDS tile is a chain of such round trips
+// otherwise).  A pixel that maps outside the image reads clamped positions and comes out as 0, like
+// base_pixel's early return; the arithmetic of the others is base_pixel's, operation for operation.
+template <int U>
+__device__ __forceinline__ void base_pixels(const float *__restrict__ img, uint32_t I, uint32_t D, float cs, float sn,
+                                            const uint32_t (&x)[U], const uint32_t (&y)[U], float (&out)[U])
+{
+    const float src_c = __fmul_rn((float)(I - 1), 0.5f);
+    const float dst_c = __fmul_rn((float)(D - 1), 0.5f);
+    const float lim = (float)(I - 1);
+    const uint32_t last = I * I - 1;
+    float rx[U], ry[U], t00[U], t01[U], t10[U], t11[U];
+    bool inside[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float px = __fsub_rn((float)x[u], dst_c);
+        const float py = __fsub_rn((float)y[u], dst_c);
+        const float sxf = __fadd_rn(__fsub_rn(__fmul_rn(px, cs), __fmul_rn(py, sn)), src_c);
+        const float syf = __fadd_rn(__fadd_rn(__fmul_rn(px, sn), __fmul_rn(py, cs)), src_c);
+        inside[u] = !(sxf < 0.0f || sxf > lim || syf < 0.0f || syf > lim);
+        const float sxc = inside[u] ? sxf : 0.0f, syc = inside[u] ? syf : 0.0f;
+        const uint32_t ix = (uint32_t)sxc, iy = (uint32_t)syc;
+        rx[u] = __fsub_rn(sxc, (float)ix);
+        ry[u] = __fsub_rn(syc, (float)iy);
+        const uint32_t i00 = ix * I + iy;
+        t00[u] = img[i00];
+        t01[u] = img[min(i00 + 1, last)];
+        t10[u] = img[min(i00 + I, last)];
+        t11[u] = img[min(i00 + I + 1, last)];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float cx = __fsub_rn(1.0f, rx[u]), cy = __fsub_rn(1.0f, ry[u]);
+        const float a = __fmul_rn(__fmul_rn(cx, cy), t00[u]);
+        const float b = __fmul_rn(__fmul_rn(cx, ry[u]), t01[u]);
+        const float c = __fmul_rn(__fmul_rn(rx[u], cy), t10[u]);
+        const float d = __fmul_rn(__fmul_rn(rx[u], ry[u]), t11[u]);
+        out[u] = inside[u] ? __fadd_rn(__fadd_rn(__fadd_rn(a, b), c), d) : 0.0f;
+    }
+}
+
 // Quotient and remainder of a dividend below 2^24: the float reciprocal's estimate is within one of the
 // quotient and is corrected (a quarter of the instructions of the general 32-bit division).
 struct RcpDivisor {
@@ -245,6 +305,8 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
     const float cs = i ? cos_t[i] : 1.0f, sn = i ? sin_t[i] : 0.0f;
     const uint32_t nq = num_rot == 1 ? 1u : 4u, nf = use_flip ? 2u : 1u;
 
+    const uint32_t probe_block = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    PROBE(kProbeRotate, probe_block, 0);
     if (i == 0 && c == 0)
         for (uint32_t n = threadIdx.x; n < N; n += blockDim.x) key[(size_t)b * N + n] = ~0ull;
     if (PACK >= 2 && threadIdx.x < 8) s_norm[threadIdx.x] = 0;
@@ -275,21 +337,57 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
         // rows and columns [lo, hi) of the base rotation: all of it, or, when only the packed operand is
         // wanted, the square that the region reaches under the eight symmetries
         const uint32_t side = hi - lo;
-        for (uint32_t cc = 0; cc < nch; ++cc)
-            for (uint32_t p = threadIdx.x; p < side * side; p += blockDim.x) {
-                const uint32_t x = lo + p / side, y = lo + p % side;
-                s_base[cc * tile + x * Dp + y] = base_pixel(img + (size_t)cc * I * I, I, D, i, cs, sn, x, y);
+        const RcpDivisor by_side(side);
+        for (uint32_t cc = 0; cc < nch; ++cc) {
+            const float *im = img + (size_t)cc * I * I;
+            // Where 8 x 8 patches cover the square with little waste, a wave takes a patch per round and a thread two
+            // pixels whose taps are all requested before the first is used: the taps of a patch lie in a dozen rows
+            // of the image whatever the angle, where 64 pixels of one row spread over up to 64 sin(angle) rows, each
+            // a cache line of its own for the gather.  Otherwise (and for the centre crop) pixel by pixel along rows.
+            const uint32_t pw = (side + 7) / 8, cells = pw * pw * 64;
+            if (i == 0 || cells * 8 > side * side * 9) {
+                for (uint32_t p = threadIdx.x; p < side * side; p += blockDim.x) {
+                    uint32_t qx, qy;
+                    by_side.divmod(p, qx, qy);
+                    s_base[cc * tile + (lo + qx) * Dp + lo + qy] = base_pixel(im, I, D, i, cs, sn, lo + qx, lo + qy);
+                }
+            } else {
+                constexpr int kFillU = 2;
+                const RcpDivisor by_pw(pw);
+                for (uint32_t t = threadIdx.x; t < cells; t += blockDim.x * kFillU) {
+                    uint32_t x[kFillU], y[kFillU];
+                    float v[kFillU];
+                    bool live[kFillU];
+#pragma unroll
+                    for (int u = 0; u < kFillU; ++u) {
+                        const uint32_t cell = t + u * blockDim.x;
+                        uint32_t px, py;
+                        by_pw.divmod(cell >> 6, px, py);
+                        const uint32_t qx = px * 8 + ((cell >> 3) & 7), qy = py * 8 + (cell & 7);
+                        live[u] = cell < cells && qx < side && qy < side;
+                        x[u] = lo + min(qx, side - 1); y[u] = lo + min(qy, side - 1);
+                    }
+                    base_pixels<kFillU>(im, I, D, cs, sn, x, y, v);
+#pragma unroll
+                    for (int u = 0; u < kFillU; ++u)
+                        if (live[u]) s_base[cc * tile + x[u] * Dp + y[u]] = v[u];
+                }
             }
+        }
         __syncthreads();
     }
+    PROBE(kProbeRotate, probe_block, 1);
     {
         // store_variants 0: none (a mapper whose distance operand is packed below never reads the variants);
         // 1: all; 2: the base rotation and its quarter turn, of which the other six are row and column
         // reversals (the update kernel reads them that way)
         const uint32_t nf_st = store_variants == 2 ? 1u : nf, nq_st = store_variants == 2 ? min(nq, 2u) : nq;
+        const RcpDivisor by_D(D);
         for (uint32_t cc = 0; cc < (store_variants ? nch : 0u); ++cc)
             for (uint32_t p = threadIdx.x; p < DD; p += blockDim.x) {
-                const uint32_t x = p / D, y = p % D;
+                uint32_t x, y;
+                if (DD <= (1u << 24)) by_D.divmod(p, x, y);        // (the reciprocal is exact below 2^24)
+                else { x = p / D; y = p % D; }
                 for (uint32_t f = 0; f < nf_st; ++f) {
                     const uint32_t xs = f ? D - 1 - x : x;
                     for (uint32_t q = 0; q < nq_st; ++q) {
@@ -305,6 +403,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
                     }
                 }
             }
+        PROBE(kProbeRotate, probe_block, 2);
         if constexpr (PACK == 1) {
             float *opnd = (float *)pk.opnd + (size_t)b * pk.rows_pad * pk.Epad;
             for (uint32_t f = 0; f < nf; ++f)
@@ -385,6 +484,7 @@ __global__ __launch_bounds__(1024) void k_rotate(const float *__restrict__ image
             }
         }
     }
+    PROBE(kProbeRotate, probe_block, 3);
 }
 
 // The base rotation and its quarter turn for images and neurons of any size (neither fits LDS): a
@@ -1184,6 +1284,8 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     __shared__ float s_fcol[kFactorColumnMax];
     const uint32_t tid = threadIdx.x;
     const uint32_t n = blockIdx.y, part = blockIdx.x;
+    const uint32_t probe_block = blockIdx.y * gridDim.x + blockIdx.x;
+    PROBE(kProbeUpdate, probe_block, 0);
     // The factor of this neuron depends on the best match, the neuron's column of the factor matrix does not: it is
     // requested with the keys (factors_t is the matrix transposed, so the column is contiguous) and waits in LDS.
     const float *__restrict__ fcol = factors_t + (size_t)n * N;
@@ -1260,8 +1362,10 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         }
     };
     load_round(j0 + tid);
+    PROBE(kProbeUpdate, probe_block, 1);
     // first minimum of the block: within a wave by DPP, then across the four waves
     wave_first_min_u64_dpp(bv, bi);
+    PROBE(kProbeUpdate, probe_block, 2);
     if ((tid & 63) == 0) { s_val[tid >> 6] = bv; s_idx[tid >> 6] = bi; }
     __syncthreads();
     bv = s_val[0]; bi = s_idx[0];
@@ -1278,6 +1382,8 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     }
 
     const float f = column_in_lds ? s_fcol[bmu] : fcol[bmu];
+
+    PROBE(kProbeUpdate, probe_block, 3);
     if (f == 0.0f) {
         // untouched neuron: its operand row stands, its norm moves to the next buffer
         if (up.Pa && part == 0 && tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], (unsigned long long)up.na_cur[n]);
@@ -1325,6 +1431,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
             }
         }
     }
+    PROBE(kProbeUpdate, probe_block, 4);
     if (up.Pa) {
         // (f depends on the block only, so every thread of the block is here)
 #pragma unroll
@@ -1334,6 +1441,7 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
         __syncthreads();
         if (tid == 0) atomicAdd((unsigned long long *)&up.na_next[n], s_val[0] + s_val[1] + s_val[2] + s_val[3]);
     }
+    PROBE(kProbeUpdate, probe_block, 5);
 }
 
 // The update of a float32 trainer on the distance operand alone: block (part, n) finds the best match like k_update,
@@ -3449,6 +3557,24 @@ int pink_hip_kernel_times(pink_hip_ctx *ctx, uint64_t *launches_out, double *ms_
     }
     return PINK_HIP_OK;
 }
+
+#ifdef PINK_PROBE
+// (measurement builds only) the stamps of kernel `kernel`: [block][wave][slot] 100 MHz clock values, 0 = never written
+int pink_hip_probe_read(uint32_t kernel, unsigned long long *host_out, int clear)
+{
+    const size_t n = (size_t)kProbeBlocks * kProbeWaves * kProbeSlots;
+    if (kernel >= kProbeKernels) return PINK_HIP_EINVAL;
+    if (hipDeviceSynchronize() != hipSuccess) return PINK_HIP_EDEVICE;
+    if (hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_probe), n * 8, (size_t)kernel * n * 8, hipMemcpyDeviceToHost) != hipSuccess)
+        return PINK_HIP_EDEVICE;
+    if (clear) {
+        std::vector<unsigned long long> z(n, 0ull);
+        if (hipMemcpyToSymbol(HIP_SYMBOL(g_probe), z.data(), n * 8, (size_t)kernel * n * 8, hipMemcpyHostToDevice) != hipSuccess)
+            return PINK_HIP_EDEVICE;
+    }
+    return PINK_HIP_OK;
+}
+#endif
 
 int pink_hip_device_info(char *buf, size_t len)
 {
