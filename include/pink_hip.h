@@ -113,6 +113,9 @@ int pink_hip_create(pink_hip_ctx **out, const pink_hip_config *cfg);
  * reference's constructors, report argument errors before the first image is seen.  Message through
  * pink_hip_last_error(NULL). */
 int pink_hip_check_config(const pink_hip_config *cfg);
+/* Frees the context.  Images that pink_hip_train(ctx, images, n, NULL) queued and that no later call has
+ * trained yet (fewer than one launch group) are discarded, not trained: call pink_hip_get_som,
+ * pink_hip_update_counts or pink_hip_synchronize first to have them applied. */
 void pink_hip_destroy(pink_hip_ctx *ctx);
 
 /* Message of the last failing call on `ctx` (or of the last failing
@@ -163,8 +166,10 @@ int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_i
  * allocates and frees nothing and clears the part of the array it uses with a kernel.  Images are
  * processed in groups of as many as fit the array (less its last KiB, which kernels that read ahead of
  * their operand may touch); PINK_HIP_EINVAL when a single image of the context
- * does not fit (the message says how many bytes it needs), PINK_HIP_ESTATE on a trainer or while
- * per-kernel timing is on (event records allocate).  All contexts on a GPU share the one array: calls
+ * does not fit (the message says how many bytes it needs), PINK_HIP_ESTATE on a trainer, while
+ * per-kernel timing is on (event records allocate), or on a context created with
+ * PINK_HIP_KERNEL_MFMA_F32 (that measurement-only kernel choice keeps its operands in buffers of the
+ * context).  All contexts on a GPU share the one array: calls
  * that overlap on the same GPU (two contexts, two streams) race; calls one after the other are fine. */
 #define PINK_HIP_STATIC_SCRATCH_BYTES (32u << 20)
 int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images,

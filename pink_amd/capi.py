@@ -7,6 +7,7 @@ if it is missing: there is no CPU fallback.  Errors returned by the library beco
 """
 import ctypes as C
 import os
+import sys
 
 import numpy as np
 
@@ -59,6 +60,16 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise PinkError(-3, "%s is missing: run `python -m pink_amd.build` (there is no CPU fallback)" % LIB_PATH)
+        # PyTorch ships a HIP runtime of its own; this library runs on the system's.  Both can live in one
+        # process, but PyTorch's must initialise first: once this library has touched the GPU, a PyTorch that
+        # initialises afterwards finds no devices.  So where PyTorch is already imported, bring it up now.
+        torch = sys.modules.get("torch")
+        if torch is not None:
+            try:
+                if torch.cuda.is_available():
+                    torch.cuda.init()
+            except Exception:       # a PyTorch without a GPU build, or no GPU: nothing to order
+                pass
         L = C.CDLL(LIB_PATH)
         vp, u32, f32p, u32p = C.c_void_p, C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_uint32)
         L.pink_hip_abi_version.restype = C.c_int

@@ -835,6 +835,8 @@ __global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__
     const float *rp = rotT + (size_t)r0 * Epad, *np = somP + (size_t)nc * Epad;
     const uint32_t chunks = Epad / kDistKC;
     float acc = 0.0f;
+    const uint32_t probe_block = blockIdx.y * gridDim.x + blockIdx.x;
+    PROBE(kProbeTrainF32, probe_block, 0);
     if (prev.key == nullptr) {
         if (stages) ssd_lone_wave_loop(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks);
         else ssd_lone_wave_loop_unstaged(acc, noff, ldsr, np, chunks);
@@ -861,6 +863,7 @@ __global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__
         const float w0 = np[lane];
         const float *xp = prev.rotT + (size_t)__builtin_amdgcn_readfirstlane((int)r) * Epad;
         const float x0 = xp[lane];
+        PROBE(kProbeTrainF32, probe_block, 1);       // everything requested (the variant's address needed the key)
         // The best match: the smallest distance of the wave (a reduction over the lanes by DPP), then the first
         // neuron that has it.
         uint32_t dmin = 0xffffffffu;
@@ -886,6 +889,7 @@ __global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__
             atomicAdd(&prev.counts[bmu], 1u);          // m_update_info[bmu]++ (Trainer.h:302-303)
         }
         float *wp = prev.somP_next + (size_t)nc * Epad;
+        PROBE(kProbeTrainF32, probe_block, 2);       // best match and factor known
         if (f == 0.0f) {
             asm volatile("" ::"v"(first0), "v"(first1), "v"(first2), "v"(first3), "v"(w0), "v"(x0));   // (requested, not used)
             if (stages) ssd_lone_wave_loop_copy(acc, roff0, roff1, roff2, roff3, noff, ldsw, ldsr, rp, np, chunks, wp);
@@ -900,8 +904,10 @@ __global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__
                                                upd + wave * 512 + (lane & 15) * 16, w0, x0);
         }
     }
+    PROBE(kProbeTrainF32, probe_block, 3);           // the chunk loop done
     const unsigned long long kv = wave_min_key_dpp(__float_as_uint(acc), r0 + lane < R, r0);
     if (lane == 0 && n < N) atomicMin(&key[n], kv);
+    PROBE(kProbeTrainF32, probe_block, 4);
 }
 
 // The same distance for large problems (many waves per SIMD): the neuron values are scalar operands.
@@ -1865,7 +1871,8 @@ struct pink_hip_ctx {
     uint32_t *d_upos = nullptr, *d_aoff = nullptr;
     unsigned char *d_kmask = nullptr;
 
-    // integer distances as an int8 MFMA GEMM with split k (training, SOMs of any size)
+    // integer distances as an int8 MFMA GEMM, one launch: every block owns an output tile over the whole k range
+    // (training, SOMs of any size)
     bool gemm = false;
     uint32_t gKS = 0, Np = 0, Rp = 0;
     bool g_tile32 = false;     // one image: a block per 32 x 32 tile instead of 64 x 64 (few tiles, long rows)
@@ -2303,6 +2310,9 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     const uint32_t target_blocks = (size_t)ctx->N * ctx->S >= ((size_t)1 << 20) ? 1024u : 128u;
     uint32_t parts = (target_blocks + ctx->N - 1) / ctx->N;
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
+#ifdef PINK_UPD_PARTS
+    parts = PINK_UPD_PARTS;
+#endif
     UpdatePlanes up{};
     if (ctx->fused_som) {
         up.Pa = (signed char *)cur_gPa(ctx);
@@ -3302,15 +3312,23 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
         // Nothing to hand back (the reference's operator() returns nothing either): the images join the
         // pending launch group in pinned memory and the call returns; see flush_pending.
         if (!ctx->pend_pin[0]) {
-            ctx->pend_cap = ctx->Bcap;
-            for (int i = 0; i < 2; ++i) {
-                if (hipHostMalloc((void **)&ctx->pend_pin[i], (size_t)ctx->pend_cap * img_bytes, hipHostMallocDefault) != hipSuccess) {
-                    ctx->pend_pin[i] = nullptr;
-                    if (i == 1) { (void)hipHostFree(ctx->pend_pin[0]); ctx->pend_pin[0] = nullptr; }
-                    return fail(ctx, PINK_HIP_ENOMEM, "pinned host allocation failed");
+            // both buffers and both events, or none of them: the context takes them only when all four exist
+            char *pin[2] = {nullptr, nullptr};
+            hipEvent_t ev[2] = {nullptr, nullptr};
+            bool ok = true;
+            for (int i = 0; i < 2 && ok; ++i)
+                ok = hipHostMalloc((void **)&pin[i], (size_t)ctx->Bcap * img_bytes, hipHostMallocDefault) == hipSuccess &&
+                     hipEventCreateWithFlags(&ev[i], hipEventDisableTiming) == hipSuccess;
+            if (!ok) {
+                (void)hipGetLastError();
+                for (int i = 0; i < 2; ++i) {
+                    if (ev[i]) (void)hipEventDestroy(ev[i]);
+                    if (pin[i]) (void)hipHostFree(pin[i]);
                 }
-                HIP_TRY(ctx, hipEventCreateWithFlags(&ctx->pend_ev[i], hipEventDisableTiming));
+                return fail(ctx, PINK_HIP_ENOMEM, "pink_hip_train: pinned host buffers for queued images could not be set up");
             }
+            ctx->pend_cap = ctx->Bcap;
+            for (int i = 0; i < 2; ++i) { ctx->pend_pin[i] = pin[i]; ctx->pend_ev[i] = ev[i]; }
         }
         for (uint32_t done = 0; done < n_images;) {
             const uint32_t take = std::min(n_images - done, ctx->pend_cap - ctx->pend_count);
@@ -3351,7 +3369,7 @@ int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_i
 {
     if (!ctx || (n_images && (!dev_images || !dev_heatmap_out)))
         return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device: null argument");
-    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map: context was created with update factors (a trainer)");
+    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device: context was created with update factors (a trainer)");
     HIP_TRY(ctx, hipSetDevice(ctx->device));
     for (uint32_t done = 0; done < n_images; done += ctx->Bcap) {
         const uint32_t B = std::min(ctx->Bcap, n_images - done);
@@ -3395,7 +3413,11 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
 {
     if (!ctx || (n_images && (!dev_images || !dev_heatmap_out)))
         return fail(ctx, PINK_HIP_EINVAL, "pink_hip_map_device_static: null argument");
-    if (ctx->trainer) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map: context was created with update factors (a trainer)");
+    if (ctx->trainer)
+        return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: context was created with update factors (a trainer)");
+    if (ctx->f32gemm)
+        return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: the float32 matrix-core kernel choice keeps its operands "
+                                          "in buffers of the context; not available through this entry point");
     if (ctx->profiling)
         return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: per-kernel timing creates events; switch it off");
     if (!ctx->static_scratch) return fail(ctx, PINK_HIP_ESTATE, "pink_hip_map_device_static: no static scratch on this device");
@@ -3421,8 +3443,7 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
     // the kernels take the scratch where they take the context's own buffers in pink_hip_map_device
     struct Saved {
         unsigned long long *key; signed char *Pb; int *nb; v4i *gPb; long long *gnb; float *rot; void *rotT;
-        uint32_t Bcap;
-    } const saved{ctx->d_key, ctx->d_Pb, ctx->d_nb, ctx->d_gPb, ctx->d_gnb, ctx->d_rot, ctx->d_rotT, ctx->Bcap};
+    } const saved{ctx->d_key, ctx->d_Pb, ctx->d_nb, ctx->d_gPb, ctx->d_gnb, ctx->d_rot, ctx->d_rotT};
     unsigned char *at = ctx->static_scratch;
     auto carve = [&](size_t bytes_per_image) { unsigned char *p = at; at += (size_t)B * bytes_per_image; return p; };
     ctx->d_key = (unsigned long long *)carve(pc.key);
@@ -3432,7 +3453,6 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
     if (pc.gnb) ctx->d_gnb = (long long *)carve(pc.gnb);
     if (pc.rot) ctx->d_rot = (float *)carve(pc.rot);
     if (pc.rotT) ctx->d_rotT = carve(pc.rotT);
-    ctx->Bcap = B;
     int rc = PINK_HIP_OK;
     for (uint32_t done = 0; done < n_images && rc == PINK_HIP_OK; done += B) {
         const uint32_t b = std::min(B, n_images - done);
@@ -3442,7 +3462,7 @@ int pink_hip_map_device_static(pink_hip_ctx *ctx, const float *dev_images, uint3
                               dev_best_rot_out ? dev_best_rot_out + (size_t)done * ctx->N : nullptr, true);
     }
     ctx->d_key = saved.key; ctx->d_Pb = saved.Pb; ctx->d_nb = saved.nb; ctx->d_gPb = saved.gPb; ctx->d_gnb = saved.gnb;
-    ctx->d_rot = saved.rot; ctx->d_rotT = saved.rotT; ctx->Bcap = saved.Bcap;
+    ctx->d_rot = saved.rot; ctx->d_rotT = saved.rotT;
     return rc;
 }
 

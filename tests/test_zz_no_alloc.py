@@ -136,7 +136,12 @@ def test_static_scratch_refusals():
         with capi.Context(4, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.UINT8, F) as tr:
             with pytest.raises(capi.PinkError) as e:
                 tr.map_device_static(imgs, 1, heat)
-            assert e.value.status == -4
+            assert e.value.status == -4 and "pink_hip_map_device_static" in str(e.value)
+        # the float32 matrix-core kernel choice (measurement only) keeps its operands in the context's own buffers
+        with capi.Context(4, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.FLOAT, kernel_choice=capi.KERNEL_MFMA_F32) as mf:
+            with pytest.raises(capi.PinkError) as e:
+                mf.map_device_static(imgs, 1, heat)
+            assert e.value.status == -4 and "float32 matrix-core" in str(e.value)
         with capi.Context(4, 1, 16, 12, 8, True, 8, capi.QUADRATIC, capi.UINT8) as mp:
             mp.set_profiling(True)
             with pytest.raises(capi.PinkError) as e:
