@@ -58,7 +58,7 @@ __device__ __forceinline__ void probe_stamp(uint32_t kernel, uint32_t block, uin
 }
 #define PROBE(kernel, block, slot) probe_stamp(kernel, block, slot)
 #else
-#define PROBE(kernel, block, slot) ((void)0)
+#define PROBE(kernel, block, slot) ((void)(kernel), (void)(block), (void)(slot))
 #endif
 constexpr uint32_t kProbeRotate = 0, kProbeGemm = 1, kProbeUpdate = 2, kProbeTrainF32 = 3;
 
@@ -2249,7 +2249,13 @@ void launch_dist_gemm(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     fin.nb = ctx->d_gnb + (size_t)slot * ctx->Rp;
     fin.variant = ctx->d_gvariant;
     fin.N = ctx->N; fin.R = ctx->R;
-    if (tile32)
+    const uint32_t real_tiles = ((ctx->R + side - 1) / side) * ((ctx->N + side - 1) / side);
+    if (tile32 && real_tiles <= (uint32_t)ctx->num_cu) {
+        // one block per CU at most: every XCD takes the same number of consecutive real tiles (see the kernel)
+        const uint32_t per_xcd = (real_tiles + 7) / 8;
+        hipLaunchKernelGGL((k_dist_gemm_int<U16, 1>), dim3(8 * per_xcd, 1), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
+                           ctx->Np, ctx->Rp, ctx->gKS, ks_per, per_xcd, 0u, 1u, fin);
+    } else if (tile32)
         hipLaunchKernelGGL((k_dist_gemm_int<U16, 1>), dim3(8 * tiles_per_xcd, 1), dim3(256), 0, ctx->stream, cur_gPa(ctx), pb,
                            ctx->Np, ctx->Rp, ctx->gKS, ks_per, rect_h, rect_w, xc, fin);
     else
