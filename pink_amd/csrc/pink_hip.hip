@@ -2771,6 +2771,10 @@ int init_ctx(pink_hip_ctx *ctx)
             const size_t stored = ctx->pair_variants ? std::min<size_t>(2 * std::max(ctx->nrr, 1u), ctx->R) : ctx->R;
             const size_t touched = per_image - (ctx->R - stored) * ctx->S * 4;
             while (b > 16 && b * touched > ((size_t)224 << 20)) b -= std::min<size_t>(8, b - 16);
+            // the integer GEMM trainers read a group's data with both of their per-image kernels and gain more from
+            // the cache than the rotation kernel loses on smaller launches (hexagonal uint16 SOM: 30.6 us per image
+            // with 16 images, 230 MB; 29.1-29.3 with 11 to 13; 29.7 with 8 to 10; 30.7 with 6)
+            if (ctx->gemm) while (b > 8 && b * touched > ((size_t)192 << 20)) --b;
         }
         ctx->Bcap = (uint32_t)b;
     } else {
