@@ -2336,7 +2336,21 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
                        is_int(ctx) ? (float)ctx->factor : 0.0f, up, ctx->d_counts, vp)
     // a slice of several rounds keeps eight elements per thread in flight (cfg2 -6 %, cfg3 -3 % against four);
     // a slice of one round is faster with four (cfg0 +8 % with eight)
-    if ((ctx->S + parts - 1) / parts > 1024) LAUNCH_UPDATE(8); else LAUNCH_UPDATE(4);
+    // ... and in rounds of equal length: a slice of 2809 elements takes two rounds of six per thread, not eight and three
+    // (cfg2: 15.2 -> 14.6 us; eleven or twelve per thread, a single round, 15.8 and 16.1)
+    const uint32_t chunk = (ctx->S + parts - 1) / parts;
+    uint32_t per_thread = 4;
+    if (chunk > 1024) {
+        const uint32_t rounds = (chunk + 2047) / 2048;
+        per_thread = std::min(8u, std::max(4u, (chunk + 256 * rounds - 1) / (256 * rounds)));
+    }
+    switch (per_thread) {
+    case 4: LAUNCH_UPDATE(4); break;
+    case 5: LAUNCH_UPDATE(5); break;
+    case 6: LAUNCH_UPDATE(6); break;
+    case 7: LAUNCH_UPDATE(7); break;
+    default: LAUNCH_UPDATE(8); break;
+    }
 #undef LAUNCH_UPDATE
     if (ctx->fused_som) ctx->na_cur ^= 1;                  // the norms of the updated SOM are in the other buffer now
     return launch_check(ctx, "k_update");
