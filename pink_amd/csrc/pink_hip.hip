@@ -919,7 +919,7 @@ __global__ __launch_bounds__(512) void k_train_f32_dpp(const float *__restrict__
 template <int TN, int KC, int MINB, int SW, bool NL>
 __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restrict__ somP, const float *__restrict__ rotT,
                                                            unsigned long long *__restrict__ key, uint32_t N, uint32_t Epad,
-                                                           uint32_t R, uint32_t Rpad)
+                                                           uint32_t R, uint32_t Rpad, uint32_t lane_tiles, uint32_t scal_groups)
 {
     static_assert(KC == 64 || KC == 32, "stage width");
     static_assert(SW == 16 || SW == 8, "slab width");
@@ -935,8 +935,14 @@ __global__ __launch_bounds__(256, MINB) void k_dist_f32_sg(const float *__restri
     // Rows on the lanes (64 per block, through LDS) and rows as scalar operands (TN per wave): rotations and
     // neurons, or (NL) neurons and rotations -- whichever wastes fewer lanes on padding.  A chain is the same
     // sequence of operations either way (the difference changes sign, its square does not).
-    const uint32_t l0 = blockIdx.x * kWave;
-    const uint32_t s0 = blockIdx.y * (4 * TN) + wave * TN;
+    // Workgroups go to the 8 XCDs round-robin by linear id and each XCD has its own L2: XCD k takes the k-th run of
+    // consecutive (lane tile, scalar group) pairs, lane tile slowest, so it streams a few lane tiles instead of all of them
+    // (the grid is padded to a multiple of 8; the blocks beyond the last pair leave at once, whole)
+    const uint32_t per_xcd = gridDim.x / 8, pair = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (pair >= lane_tiles * scal_groups) return;
+    const uint32_t lane_tile = pair / scal_groups, scal_group = pair - lane_tile * scal_groups;
+    const uint32_t l0 = lane_tile * kWave;
+    const uint32_t s0 = scal_group * (4 * TN) + wave * TN;
     const float *laneP = NL ? somP : rotT + (size_t)b * Rpad * Epad;
     const float *scalP = NL ? rotT + (size_t)b * Rpad * Epad : somP;
     const uint32_t lane_rows = NL ? N : Rpad;             // rows that exist on the lane side (loads are clamped to them)
@@ -2209,10 +2215,12 @@ void launch_dist_f32(pink_hip_ctx *ctx, uint32_t slot, uint32_t B)
     const bool neurons_on_lanes = work_neu * 100 < work_rot * 98;
     const uint32_t lane_blocks = neurons_on_lanes ? nblocks : rblocks, scal_rows = neurons_on_lanes ? ctx->R : ctx->N;
     const uint32_t tn = (size_t)lane_blocks * groups(scal_rows, 4) * B >= (size_t)4 * ctx->num_cu ? 4 : 2;
-    const dim3 grid(lane_blocks, groups(scal_rows, tn), B);
+    const uint32_t scal_groups = groups(scal_rows, tn);
+    const dim3 grid((lane_blocks * scal_groups + 7) / 8 * 8, 1, B);        // (see the kernel: an XCD takes a run of pairs)
 #define LAUNCH_SG(...)                                                                                             \
     hipLaunchKernelGGL((k_dist_f32_sg<__VA_ARGS__>), grid, dim3(256), 0, ctx->stream, (const float *)ctx->d_somP,  \
-                       (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad, key, ctx->N, ctx->Epad, ctx->R, ctx->Rpad)
+                       (const float *)ctx->d_rotT + (size_t)slot * ctx->Epad * ctx->Rpad, key, ctx->N, ctx->Epad, ctx->R, ctx->Rpad, \
+                       lane_blocks, scal_groups)
     // (TN = 4: 8-element slabs, 4 x 8 x 2 sets of scalar registers)
     if (neurons_on_lanes) { if (tn == 4) LAUNCH_SG(4, 32, 6, 8, true); else LAUNCH_SG(2, 32, 6, 16, true); }
     else { if (tn == 4) LAUNCH_SG(4, 32, 6, 8, false); else LAUNCH_SG(2, 32, 6, 16, false); }
