@@ -2324,9 +2324,6 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     const uint32_t target_blocks = (size_t)ctx->N * ctx->S >= ((size_t)1 << 20) ? 1024u : 128u;
     uint32_t parts = (target_blocks + ctx->N - 1) / ctx->N;
     parts = std::max(1u, std::min(parts, (ctx->S + 255) / 256));
-#ifdef PINK_UPD_PARTS
-    parts = PINK_UPD_PARTS;
-#endif
     UpdatePlanes up{};
     if (ctx->fused_som) {
         up.Pa = (signed char *)cur_gPa(ctx);
