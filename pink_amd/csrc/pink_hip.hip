@@ -31,7 +31,10 @@
 #include <type_traits>
 #include <vector>
 
+#include <condition_variable>
+#include <memory>
 #include <mutex>
+#include <thread>
 
 #include "mfma_u8_sym.h"
 #include "pink_hip.h"
@@ -1797,6 +1800,74 @@ __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__re
 // Host side
 // ---------------------------------------------------------------------------------
 struct EventPair { hipEvent_t a, b; int cls; uint32_t launches; };
+
+// Host threads that copy one buffer into another side by side (the caller takes a part too): what carries a large
+// pageable input of a mapper into pinned memory faster than one thread can (a single thread moves about half of what the
+// PCIe link takes).  copy() returns when every part has been copied.
+class HostCopyPool {
+public:
+    explicit HostCopyPool(unsigned workers)
+    {
+        for (unsigned i = 0; i < workers; ++i) threads_.emplace_back([this, i] { loop(i); });
+    }
+    ~HostCopyPool()
+    {
+        {
+            std::lock_guard<std::mutex> lock(m_);
+            stop_ = true;
+            ++generation_;
+        }
+        start_.notify_all();
+        for (std::thread &t : threads_) t.join();
+    }
+    void copy(char *dst, const char *src, size_t bytes)
+    {
+        const size_t parts = threads_.size() + 1;
+        {
+            std::lock_guard<std::mutex> lock(m_);
+            dst_ = dst; src_ = src; bytes_ = bytes;
+            each_ = ((bytes + parts - 1) / parts + 4095) & ~(size_t)4095;
+            pending_ = (unsigned)threads_.size();
+            ++generation_;
+        }
+        start_.notify_all();
+        part((unsigned)threads_.size());
+        std::unique_lock<std::mutex> lock(m_);
+        done_.wait(lock, [&] { return pending_ == 0; });
+    }
+
+private:
+    void part(unsigned i) const
+    {
+        const size_t off = (size_t)i * each_;
+        if (off < bytes_) memcpy(dst_ + off, src_ + off, std::min(each_, bytes_ - off));
+    }
+    void loop(unsigned i)
+    {
+        unsigned long long seen = 0;
+        for (;;) {
+            {
+                std::unique_lock<std::mutex> lock(m_);
+                start_.wait(lock, [&] { return generation_ != seen; });
+                seen = generation_;
+                if (stop_) return;
+            }
+            part(i);
+            std::lock_guard<std::mutex> lock(m_);
+            if (--pending_ == 0) done_.notify_one();
+        }
+    }
+    std::vector<std::thread> threads_;
+    std::mutex m_;
+    std::condition_variable start_, done_;
+    unsigned long long generation_ = 0;
+    unsigned pending_ = 0;
+    bool stop_ = false;
+    char *dst_ = nullptr;
+    const char *src_ = nullptr;
+    size_t bytes_ = 0, each_ = 0;
+};
+constexpr size_t kBounceBytes = (size_t)8 << 20;          // pinned buffers the pool fills, two taking turns
 constexpr size_t kRotateLdsMax = 158 * 1024;
 enum : uint32_t { kStoreNone = 0, kStoreAll = 1, kStorePair = 2 };
 
@@ -1860,6 +1931,10 @@ struct pink_hip_ctx {
     uint32_t pend_count = 0, pend_cur = 0, pend_cap = 0;
     hipStream_t copy_stream = nullptr;     // host -> device copies of the next images while the kernels of the last run
     hipEvent_t copy_ev[2] = {};
+    // mappers, large pageable inputs: host threads fill two pinned buffers in turn, the copies to the device leave from those
+    std::unique_ptr<HostCopyPool> copy_pool;
+    char *bounce[2] = {nullptr, nullptr};
+    hipEvent_t bounce_ev[2] = {};
     uint32_t *d_counts = nullptr;          // trainer: how often each neuron was the best match
     uint32_t *d_symoff = nullptr;          // [8][Epad] region positions under the 8 symmetries: packing fused into k_rotate
     bool fused_pack = false;
@@ -2479,6 +2554,12 @@ int free_all(pink_hip_ctx *ctx)
     }
     for (hipEvent_t e : ctx->st_ev) if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : ctx->copy_ev) if (e) (void)hipEventDestroy(e);
+    ctx->copy_pool.reset();
+    for (int i = 0; i < 2; ++i) {
+        if (ctx->bounce[i]) (void)hipHostFree(ctx->bounce[i]);
+        if (ctx->bounce_ev[i]) (void)hipEventDestroy(ctx->bounce_ev[i]);
+        ctx->bounce[i] = nullptr; ctx->bounce_ev[i] = nullptr;
+    }
     if (ctx->copy_stream) (void)hipStreamDestroy(ctx->copy_stream);
     if (ctx->d_counts) (void)hipFree(ctx->d_counts);
     for (void *p : {(void *)ctx->d_fPa, (void *)ctx->d_fPb, (void *)ctx->d_fna, (void *)ctx->d_fnb, (void *)ctx->d_fpart})
@@ -3316,10 +3397,50 @@ int staged_run(pink_hip_ctx *ctx, const float *host_images, uint32_t n, Run run)
     };
     const uint32_t largest = whole_groups((size_t)(ctx->trainer ? 16 : 64) << 20);
     uint32_t piece = std::min(largest, std::max(whole_groups((size_t)1 << 20), std::min(ctx->Bcap, largest)));
-    uint32_t turn = 0, count = 0;
+    // A mapper's kernels are faster than the link, so its rate from host buffers is the rate of the copies, and a
+    // copy out of pageable memory is one host thread's work (about half of what the link takes): inputs of 32 MB and
+    // more go through two pinned buffers that four host threads fill side by side (cfg1 from pageable memory: 26 -> 42 GB/s,
+    // 1.6 M -> 2.56 M images/s).
+    // Set up all or nothing; a host that cannot give the threads or the pinned memory keeps the plain copies.
+    const bool pooled = !ctx->trainer && (size_t)n * img_bytes >= ((size_t)32 << 20);
+    if (pooled && !ctx->copy_pool) {
+        char *pin[2] = {nullptr, nullptr};
+        hipEvent_t ev[2] = {nullptr, nullptr};
+        bool ok = true;
+        for (int i = 0; i < 2 && ok; ++i)
+            ok = hipHostMalloc((void **)&pin[i], kBounceBytes, hipHostMallocDefault) == hipSuccess &&
+                 hipEventCreateWithFlags(&ev[i], hipEventDisableTiming) == hipSuccess;
+        std::unique_ptr<HostCopyPool> pool;
+        if (ok) {
+            // (three workers and the caller; five or seven workers, buffers of 4 or 16 MB: the same 42 GB/s)
+            try { pool.reset(new HostCopyPool(3)); } catch (...) { ok = false; }
+        }
+        if (ok) {
+            ctx->copy_pool = std::move(pool);
+            for (int i = 0; i < 2; ++i) { ctx->bounce[i] = pin[i]; ctx->bounce_ev[i] = ev[i]; }
+        } else {
+            (void)hipGetLastError();
+            for (int i = 0; i < 2; ++i) {
+                if (ev[i]) (void)hipEventDestroy(ev[i]);
+                if (pin[i]) (void)hipHostFree(pin[i]);
+            }
+        }
+    }
+    uint32_t turn = 0, count = 0, bounce_turn = 0;
     for (uint32_t first = 0; first < n; first += count, turn ^= 1, piece = std::min(largest, 2 * piece)) {
         count = std::min(piece, n - first);
         float *dev = ctx->st_img + (size_t)first * ctx->isz;
+        if (pooled && ctx->copy_pool) {
+            const char *src = (const char *)(host_images + (size_t)first * ctx->isz);
+            const size_t bytes = (size_t)count * img_bytes;
+            for (size_t off = 0; off < bytes; off += kBounceBytes, bounce_turn ^= 1) {
+                const size_t len = std::min(kBounceBytes, bytes - off);
+                HIP_TRY(ctx, hipEventSynchronize(ctx->bounce_ev[bounce_turn]));       // its last copy to the device has run
+                ctx->copy_pool->copy(ctx->bounce[bounce_turn], src + off, len);
+                HIP_TRY(ctx, hipMemcpyAsync((char *)dev + off, ctx->bounce[bounce_turn], len, hipMemcpyHostToDevice, ctx->copy_stream));
+                HIP_TRY(ctx, hipEventRecord(ctx->bounce_ev[bounce_turn], ctx->copy_stream));
+            }
+        } else
         HIP_TRY(ctx, hipMemcpyAsync(dev, host_images + (size_t)first * ctx->isz, count * img_bytes, hipMemcpyHostToDevice,
                                     ctx->copy_stream));
         HIP_TRY(ctx, hipEventRecord(ctx->copy_ev[turn], ctx->copy_stream));

@@ -601,8 +601,10 @@ def test_map_full_size_properties():
 
 
 def test_host_buffers_in_pieces_match_smaller_calls():
-    """Inputs beyond 64 MB go to the device piece by piece while the kernels of the piece before run:
-    the results are those of calls small enough to go in one piece."""
+    """Inputs beyond 64 MB go to the device piece by piece while the kernels of the piece before run, a mapper's
+    inputs from 32 MB on through two pinned buffers that several host threads fill side by side (147 MB here: pieces
+    that are no multiple of the 8 MB buffers): the results are those of calls small enough to go in one plain copy
+    (1500 images, 25 MB)."""
     w = synthetic.WORKLOADS["cfg1"]
     n = 9000                                                   # 147 MB of images: three pieces
     imgs = synthetic.images(w, n)
