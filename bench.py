@@ -48,15 +48,15 @@ MEASURED_VALU_LANE_OPS_T = 50.0     # subtract / fma stream, eight waves per SIM
 # under profiles/ that holds the readings).  Not measured in the run that prints the line.
 COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg0", "distance"): (12.280e6 + 3.239e6, "profiles/cfg0_train_f32_counters.txt"),   # with the update of the image before
-    ("cfg0", "update"): ((28.149e6 + 0.774e6 + 1.711e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
-    ("cfg1", "rotate"): ((95.405e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg1", "distance"): ((214.632e6 + 1.640e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
-    ("cfg2", "distance"): (25.224e6 + 0.070e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg2", "update"): (27.032e6 + 20.729e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (874.783e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg0", "update"): ((28.133e6 + 0.774e6 + 1.706e6 + 1.184e6) / 48, "profiles/cfg0_train_f32_counters.txt"),   # per group of 48
+    ("cfg1", "rotate"): ((96.042e6 + 207.618e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg1", "distance"): ((214.632e6 + 1.639e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
+    ("cfg2", "distance"): (33.018e6 + 0.069e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg2", "update"): (26.987e6 + 20.737e6, "profiles/cfg2_train_u16_counters.txt"),
+    ("cfg3", "distance"): (247.797e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
-    ("cfg3", "update"): (73.898e6 + 47.153e6 + (294.770e6 + 94.546e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg4", "update"): (1.205e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
+    ("cfg3", "update"): (73.892e6 + 47.153e6 + (295.051e6 + 94.661e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg4", "update"): (1.231e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
 }
 
 # Images per step of the workloads that ride along in `all_configs` (the headline workload always

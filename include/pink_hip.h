@@ -151,7 +151,9 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
 
 /* Mapper<...,true>::operator()(Data const&) (Mapper.h:181-208) for n_images images:
  * heatmap_out[i*N + n] = sqrt(min over rotations of the distance), already square-rooted
- * (Mapper.h:206); best_rot_out[i*N + n] = index of that rotation (may be NULL). */
+ * (Mapper.h:206); best_rot_out[i*N + n] = index of that rotation (may be NULL).
+ * A call that brings 32 MB of images or more starts three helper threads in the context (kept until
+ * pink_hip_destroy) that copy the input into pinned memory beside the calling thread. */
 int pink_hip_map(pink_hip_ctx *ctx, const float *host_images, uint32_t n_images,
                  float *host_heatmap_out, uint32_t *host_best_rot_out);
 int pink_hip_map_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images,
