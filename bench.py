@@ -148,10 +148,13 @@ def cpu_baseline(w, som0, imgs_host, budget_s, quick=False):
         O.set_num_threads(nthreads)
         try:
             n_all = len(imgs_host)
-            probe = run(s, 1)                              # warm-up, and how long an image takes
+            probe = run(s, 1)                              # warm-up, and roughly how long an image takes
             n, dt = 1, probe
             if probe < budget / 2:
-                n = int(max(1, min(n_all, budget / max(probe, 1e-6))))
+                # (the first image also wakes the thread pool: a second, warm probe sizes the sample)
+                n = int(max(1, min(n_all, 0.1 * budget / max(probe, 1e-6))))
+                dt = run(s, n)
+                n = int(max(1, min(n_all, budget / max(dt / n, 1e-6))))
                 dt = run(s, n)
         finally:
             O.set_num_threads(threads)
