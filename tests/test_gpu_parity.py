@@ -104,8 +104,6 @@ def _som_and_image(N, C_, I, D, seed):
 @pytest.mark.parametrize("ed_type", [capi.FLOAT, capi.UINT8, capi.UINT16])
 @pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_", DIST_SHAPES)
 def test_distance_parity(N, C_, I, D, nrot, flip, ed, shape_, ed_type):
-    if N >= 331 and ed_type != {331: capi.UINT16, 1600: capi.FLOAT}[N]:
-        pytest.skip("large shapes run in their configured mode only (oracle time)")
     say("distance", N, C_, I, D, nrot, flip, ed, shape_, ed_type)
     som, img = _som_and_image(N, C_, I, D, N + D + ed)
     if N < 331:
