@@ -274,16 +274,22 @@ class InputData:
             raise UsageError("Periodic boundary conditions are not supported in version 2.")
         if not self.use_gpu:
             raise UsageError("this build has no CPU path: --cuda-off is not supported")
-        if self.som_depth != 1:
-            raise UsageError("three-dimensional SOM layouts are not supported by this build")
         return self
 
     # -- objects of the path ------------------------------------------------------------------------
+    def som_dimensionality(self):
+        """InputData.cpp:429-430: one, plus one for a height above 1, plus one for a depth above 1; the SOM
+        then takes that many of (width, height, depth) in this order (SOM.h:25-43,71-72), so a height of 1
+        with a depth above 1 gives a width x 1 SOM, as in the reference."""
+        return 1 + (self.som_height > 1) + (self.som_depth > 1)
+
     def som_layout(self):
-        return "hexagonal-2d" if self.layout == "hexagonal" else "cartesian-2d"
+        return "hexagonal-2d" if self.layout == "hexagonal" else "cartesian-%dd" % self.som_dimensionality()
 
     def som_dims(self):
-        return (self.som_width,) if self.layout == "hexagonal" else (self.som_width, self.som_height)
+        if self.layout == "hexagonal":
+            return (self.som_width,)
+        return (self.som_width, self.som_height, self.som_depth)[:self.som_dimensionality()]
 
     def neuron_layout(self):
         return "cartesian-3d" if len(self.neuron_dimension) == 3 else "cartesian-2d"
@@ -308,7 +314,7 @@ def run(argv):
                                  cfg.som_filename)
     shape = ((cfg.som_size,) if cfg.layout == "hexagonal" else cfg.som_dims()) + tuple(cfg.neuron_dimension)
     som = pink.SOM(np.ascontiguousarray(weights).reshape(shape), som_layout=cfg.som_layout(),
-                   neuron_layout=cfg.neuron_layout())
+                   neuron_layout=cfg.neuron_layout(), _command_line=True)
     common = dict(verbosity=int(cfg.verbose), number_of_rotations=cfg.number_of_rotations, use_flip=cfg.use_flip,
                   interpolation=cfg.interpolation, euclidean_distance_dim=cfg.euclidean_distance_dim,
                   euclidean_distance_shape=cfg.euclidean_distance_shape,

@@ -14,6 +14,9 @@ What differs from the reference module:
   * `use_gpu=False` raises: this build has no CPU path (the reference's CPU classes are its own);
   * `Trainer.train(images)` / `Mapper.map(images)` take a whole array of images per call (the
     per-image `__call__` costs one host round trip per image, as in the reference);
+  * SOM layouts: "cartesian-2d" and "hexagonal-2d" as in the reference's module (src/pink/DynamicSOM.cpp:22-42);
+    "cartesian-1d" and "cartesian-3d" only for this package's command line (`_command_line=True`), whose
+    counterpart in the reference builds such SOMs directly (CudaLib/main_gpu.cu:19-25);
   * neuron layouts: "cartesian-2d" (edge, edge) and "cartesian-3d" (channels, edge, edge); the
     reference's spatial transformer throws for "cartesian-1d"
     (SelfOrganizingMapLib/generate_rotated_images.h:36-46), so does this module.
@@ -132,15 +135,17 @@ class SOM:
     """pink.SOM (src/pink/DynamicSOM.cpp:12-44): shape = SOM dimensions followed by the neuron
     shape; "hexagonal-2d" takes the number of neurons as its one SOM dimension."""
 
-    def __init__(self, buffer, data_type="float32", som_layout="cartesian-2d", neuron_layout="cartesian-2d"):
+    def __init__(self, buffer, data_type="float32", som_layout="cartesian-2d", neuron_layout="cartesian-2d",
+                 _command_line=False):
         if data_type != "float32":
             raise exception(-1, "data-type not supported")
         self._a = _as_float32_copy(buffer, "som")
         shape = self._a.shape
-        if som_layout == "cartesian-2d":
-            if len(shape) < 3:
+        if som_layout == "cartesian-2d" or (_command_line and som_layout in ("cartesian-1d", "cartesian-3d")):
+            rank = int(som_layout[10])
+            if len(shape) < rank + 1:
                 raise exception(-1, "som shape does not match layout " + som_layout)
-            self._layout, self._dims, neuron_shape = capi.CARTESIAN, [shape[0], shape[1]], shape[2:]
+            self._layout, self._dims, neuron_shape = capi.CARTESIAN, list(shape[:rank]), shape[rank:]
         elif som_layout == "hexagonal-2d":
             if len(shape) < 2:
                 raise exception(-1, "som shape does not match layout " + som_layout)
@@ -299,7 +304,7 @@ class Mapper:
                  euclidean_distance_type=DataType.UINT8):
         if som.neuron_layout != "cartesian-2d" and som.neuron_layout != "cartesian-3d":
             raise exception(-1, "neuron layout " + som.neuron_layout + " is not supported")
-        snapshot = SOM(np.asarray(som), som.data_type, som.som_layout, som.neuron_layout)
+        snapshot = SOM(np.asarray(som), som.data_type, som.som_layout, som.neuron_layout, _command_line=True)
         self._dev = _Device(snapshot, number_of_rotations, use_flip, interpolation, use_gpu, euclidean_distance_dim,
                             euclidean_distance_shape, euclidean_distance_type, None)
         self.verbosity = verbosity

@@ -57,6 +57,23 @@ def test_options(tmp_path):
         assert c.max_number_of_progress_prints == want
 
 
+def test_som_dimensionality_follows_height_and_depth(tmp_path):
+    """InputData.cpp:429-430 counts a SOM dimension for the width, one for a height above 1 and one for a depth
+    above 1; the SOM takes that many of (width, height, depth) (SOM.h:25-43)."""
+    _data(tmp_path)
+    base = ["--train", str(tmp_path / "data.bin"), "x.bin"]
+    c = cli.InputData().parse(base + ["--som-width", "4", "--som-height", "3", "--som-depth", "2"]).finish()
+    assert (c.som_size, c.som_layout(), c.som_dims()) == (24, "cartesian-3d", (4, 3, 2))
+    c = cli.InputData().parse(base + ["--som-width", "7", "--som-height", "1"]).finish()
+    assert (c.som_size, c.som_layout(), c.som_dims()) == (7, "cartesian-1d", (7,))
+    # a height of 1 with a depth above 1 is two-dimensional to the reference: width x 1
+    c = cli.InputData().parse(base + ["--som-width", "5", "--som-height", "1", "--som-depth", "3"]).finish()
+    assert (c.som_layout(), c.som_dims()) == ("cartesian-2d", (5, 1))
+    with pytest.raises(cli.UsageError) as e:
+        cli.InputData().parse(base + ["-l", "hexagonal", "--som-width", "5", "--som-height", "5", "--som-depth", "2"]).finish()
+    assert "For hexagonal layout som-depth must be equal to 1." in str(e.value)
+
+
 @pytest.mark.parametrize("argv,text", [
     ([], "Unknown execution path."),
     (["--train", "DATA"], "Missing arguments for --train option."),
@@ -110,3 +127,44 @@ def test_train_then_map_from_the_command_line(tmp_path):
     _, flips, _ = fileio.read_rot_flip_file(tmp_path / "rot.bin")
     assert np.array_equal(flips, obest // 8)
     assert cli.main(["--map", data, str(tmp_path / "map.bin")]) == 1          # reports, does not raise
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dims", [(3, 2, 2), (5,)])
+def test_train_then_map_one_and_three_dimensional_soms(tmp_path, dims):
+    """--som-depth above 1 and --som-height 1: the reference's command line builds CartesianLayout<3> and <1>
+    SOMs (CudaLib/main_gpu.cu:19-25); the layout only enters through the neurons' distances
+    (CartesianLayout.h:84-123) and the file headers."""
+    images = _data(tmp_path, n=7, edge=12, seed=9)
+    data, som_file = str(tmp_path / "data.bin"), str(tmp_path / "som.bin")
+    whd = list(dims) + [1] * (3 - len(dims))
+    size = ["--som-width", str(whd[0]), "--som-height", str(whd[1]), "--som-depth", str(whd[2])]
+    assert cli.main(["--train", data, som_file] + size + ["-n", "4", "-x", "random", "-s", "3", "--input-shuffle-off",
+                                                          "--euclidean-distance-type", "float"]) == 0
+    n = int(np.prod(dims))
+    F = capi.make_update_factors(capi.CARTESIAN, list(dims), capi.GAUSSIAN, 1.1, 0.2)
+    # the distances behind F are the reference's: sqrt of the summed squared position differences, positions
+    # as CartesianLayout<N>::get_position gives them
+    D = capi.layout_distances(capi.CARTESIAN, list(dims))
+    if len(dims) == 3:
+        def pos(i):
+            z = i // dims[0] // dims[1]
+            return (i % dims[1], (i - z * dims[0] * dims[1]) // dims[1], z)
+    else:
+        def pos(i):
+            return (i,)
+    want_D = np.array([[np.sqrt(np.float32(sum((a - b) ** 2 for a, b in zip(pos(i), pos(j))))) for j in range(n)]
+                       for i in range(n)], np.float32)
+    assert np.array_equal(D.reshape(n, n), want_D)
+    s = O.shape(n, 1, 12, 17, 4, True, 8, O.QUADRATIC, capi.FLOAT)      # neuron 2 * 12 / sqrt(2) + 1 = 17, region 8
+    want = O.fill_random_uniform(n * 17 * 17, 3).reshape(n, -1)
+    O.train(s, want, images[:, None], F)
+    _, som_dims, neuron_dims, got = fileio.read_som_file(som_file)
+    assert som_dims == list(dims) and neuron_dims == [17, 17]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert cli.main(["--map", data, str(tmp_path / "map.bin"), som_file] + size + ["-n", "4", "--euclidean-distance-type",
+                                                                                  "float"]) == 0
+    oheat, _ = O.map_images(s, want, images[:, None])
+    map_dims, heat = fileio.read_mapping_file(tmp_path / "map.bin")
+    assert map_dims == list(dims)
+    assert np.array_equal(heat.view(np.uint32), oheat.view(np.uint32))
