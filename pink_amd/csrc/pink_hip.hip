@@ -51,7 +51,7 @@ static __device__ __align__(256) unsigned char scratch[PINK_HIP_STATIC_SCRATCH_B
 // none): wave w of block b of kernel k stores the 100 MHz constant clock at the places marked
 // PROBE(k, b, slot); pink_hip_probe_read copies the stamps of the last launch of each kernel out.
 #ifdef PINK_PROBE
-constexpr uint32_t kProbeKernels = 4, kProbeBlocks = 2048, kProbeWaves = 8, kProbeSlots = 8;
+constexpr uint32_t kProbeKernels = 5, kProbeBlocks = 2048, kProbeWaves = 8, kProbeSlots = 8;
 static __device__ unsigned long long g_probe[kProbeKernels * kProbeBlocks * kProbeWaves * kProbeSlots];
 __device__ __forceinline__ void probe_stamp(uint32_t kernel, uint32_t block, uint32_t slot)
 {
@@ -63,7 +63,7 @@ __device__ __forceinline__ void probe_stamp(uint32_t kernel, uint32_t block, uin
 #else
 #define PROBE(kernel, block, slot) ((void)(kernel), (void)(block), (void)(slot))
 #endif
-constexpr uint32_t kProbeRotate = 0, kProbeGemm = 1, kProbeUpdate = 2, kProbeTrainF32 = 3;
+constexpr uint32_t kProbeRotate = 0, kProbeGemm = 1, kProbeUpdate = 2, kProbeTrainF32 = 3, kProbeResident = 4;
 
 namespace {
 
@@ -1771,6 +1771,245 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
     if (tid == 0) a.na_next[n] = (long long)s_sq[0] + s_sq[1] + s_sq[2] + s_sq[3];
 }
 
+// ---------------------------------------------------------------------------------
+// The same trainers with the kernel RESIDENT over a whole launch group: one block per neuron keeps its neuron
+// -- weights in registers, its row of the SOM operand and the norm in LDS -- over all images of the group and
+// computes only its own neuron's distances (the MFMA's 32 columns all hold the one neuron).  Per image the
+// blocks exchange one 64-bit word each, (tag, smallest distance of the neuron), through slots a cache line
+// apart: a block stores its word and its first wave polls the N slots until all carry the image's tag.  Nothing
+// else crosses between blocks, so no fences: the payload rides in the atomic word.  Two sets of slots take turns
+// (a block can be at most one image ahead of another).  The exchange costs about 1.4 us, where a launch boundary
+// with the distance matrix worked out again in every block costs 5.
+// Every wait is bounded: a wave that does not see all words within `spin_limit` polls raises `error`, polling
+// waves leave when they see it raised, a block that leaves stops publishing, so every block leaves.  The group's
+// results go to the OTHER buffers (weights, operand, norms); the host looks at `error` after the launch and only
+// then makes them the current ones, or trains the group again, image by image, from the untouched current ones.
+// ---------------------------------------------------------------------------------
+constexpr uint32_t kSlotStride = 16;                      // 64-bit words between two blocks' slots (128 bytes)
+constexpr uint32_t kSlotWords = 2 * 64 * kSlotStride;     // two sets of 64 slots
+
+struct ResidentTrain {
+    const long long *na_cur;
+    long long *na_next;
+    const long long *nb;            // norms of the variant rows, first image; nb_stride apart
+    const uint32_t *variant;        // operand row -> variant index
+    uint32_t *bmu_out;              // one per image
+    unsigned long long *slots;
+    uint32_t *error;
+    uint32_t N, S, R, KS, nstored, images, tag0, spin_limit;
+    uint32_t rot_stride, pb_stride, nb_stride;      // per image: floats, 16-byte words, norms
+    VariantPair vp;
+};
+
+// Eight waves per block: two share a SIMD without slowing each other, so each wave's part of every step is half as long.
+constexpr uint32_t kResidentThreads = 512, kResidentWaves = kResidentThreads / 64;
+
+template <int EPT, int KSW, int SV>    // elements of the neuron, k-steps and variant elements (first batch) per thread
+__global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__restrict__ som, float *__restrict__ som_next,
+                                                                 const float *__restrict__ rot, const v4i *__restrict__ Pa,
+                                                                 signed char *__restrict__ Pa_next, const v4i *__restrict__ Pb,
+                                                                 const float *__restrict__ factors,
+                                                                 const unsigned long long *__restrict__ src4,
+                                                                 const uint32_t *__restrict__ kbyte, ResidentTrain a)
+{
+    extern __shared__ float s_var[];                      // the stored variants of this image and of the next one
+    __shared__ v4i s_op[128 + 1];                         // this neuron's operand row: [k-step][half of the k-step]; one spare
+    __shared__ v4i s_part[kResidentWaves][2][4];          // [wave][half][16 accumulators]
+    __shared__ float s_f[64];
+    __shared__ int s_sq[kResidentWaves];
+    __shared__ uint32_t s_bmu;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = blockIdx.x;
+    const uint32_t N = a.N, S = a.S, KS = a.KS, n_var = a.nstored * S;
+    // (a launch that follows one that gave up leaves at once; one thread looks, so the whole block decides alike)
+    if (tid == 0) s_bmu = __hip_atomic_load(a.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_bmu) return;
+
+    // what stays for the whole group
+    float wv[EPT];
+    uint32_t cb[EPT], in_region[EPT];
+    unsigned long long sp[EPT];
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        const uint32_t j = min(tid + kResidentThreads * u, S - 1);     // (past the end: the last element again, dropped at the end)
+        wv[u] = som[(size_t)n * S + j];
+        // byte inside the neuron's row of 32-row fragments, lanes 16 bytes apart; here inside s_op.  Elements outside
+        // the region (and past the end) write the spare bytes and count nothing: no branches in the update
+        const uint32_t kb = tid + kResidentThreads * u < S ? kbyte[j] : 0xffffffffu;
+        in_region[u] = kb == 0xffffffffu ? 0u : 0xffffffffu;
+        cb[u] = kb == 0xffffffffu ? 128u * 16u + (tid & 15u) : ((kb >> 9) << 4) | (kb & 15u);
+        sp[u] = src4[j];
+    }
+    if (tid < 64) s_f[tid] = tid < N ? factors[(size_t)tid * N + n] : 0.0f;
+    // (k-steps past the end hold zeros: a wave whose share of the k-steps ends early multiplies by them)
+    if (tid < 128) {
+        const v4i zero = {0, 0, 0, 0};
+        s_op[tid] = tid < 2 * KS ? Pa[((size_t)(n >> 5) * KS + (tid >> 1)) * 64 + (tid & 1) * 32 + (n & 31)] : zero;
+    }
+    int na = (int)a.na_cur[n];
+    const uint32_t row = lane & 31;                       // the operand row whose key this lane works out
+    const uint32_t var_row = a.variant[row];
+    const uint32_t acc_half = (row >> 2) & 1, acc_j = ((row >> 3) << 2) | (row & 3);     // where the MFMA leaves row `row`
+    for (uint32_t t = tid; t < n_var; t += kResidentThreads) s_var[t] = rot[t];
+    // variant r of an image: which stored variant it is read from and how (rows / columns reversed), worked out once
+    // by lane r: offset of the stored variant in floats << 8 | shift into the packed source positions
+    uint32_t dec_lane;
+    {
+        const uint32_t flip = row >= a.vp.num_rot ? 1u : 0u, rem = row - flip * a.vp.num_rot;
+        const uint32_t q = rem / a.vp.nrr, b0 = rem - q * a.vp.nrr;
+        dec_lane = ((((q & 1) * a.vp.nrr + b0) * S) << 8) | (16 * (2 * (flip ^ (q >> 1)) + (q >> 1)));
+    }
+    v4i fb[KSW];
+    auto load_fragments = [&](const v4i *pb, uint32_t first) {
+#pragma unroll
+        for (int u = 0; u < KSW; ++u) fb[u] = pb[(size_t)min(first + kResidentWaves * u, KS - 1) * 64 + lane];
+    };
+    load_fragments(Pb, wave);
+    int nb_row = (int)a.nb[row];
+    // the variants of the image after next wait in registers for a whole image (asked for during one exchange,
+    // put into LDS during the next)
+    float sv[SV];
+    auto load_variants = [&](const float *src) {
+#pragma unroll
+        for (int u = 0; u < SV; ++u) sv[u] = src[min(tid + kResidentThreads * u, n_var - 1)];
+    };
+    if (a.images > 1) load_variants(rot + a.rot_stride);
+    __syncthreads();
+
+    for (uint32_t i = 0; i < a.images; ++i) {
+        const bool more = i + 1 < a.images;
+        const v4i *pb = Pb + (size_t)i * a.pb_stride;
+        float *var_cur = s_var + (i & 1) * n_var, *var_next = s_var + ((i + 1) & 1) * n_var;
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 0);
+
+        // (1) this neuron against all variants: this wave's k-steps (the operand row out of LDS first: a lone
+        // wave waits out every LDS read it issues between two MFMAs)
+        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (uint32_t first = wave; first < KS; first += kResidentWaves * KSW) {
+            if (first != wave) load_fragments(pb, first);
+            v4i fa[KSW];
+#pragma unroll
+            for (int u = 0; u < KSW; ++u) fa[u] = s_op[min(first + kResidentWaves * u, 63u) * 2 + (lane >> 5)];
+#pragma unroll
+            for (int u = 0; u < KSW; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[u], fa[u], acc, 0, 0, 0);
+        }
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 1);
+        if ((lane & 31) == 0) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                s_part[wave][lane >> 5][g] = (v4i){acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+        }
+        __syncthreads();
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 2);
+
+        // (2) the neuron's key (every wave for itself) and its word into the exchange
+        const int *part = (const int *)&s_part[0][acc_half][0] + acc_j;
+        int dot = 0;                                          // the waves' k ranges
+#pragma unroll
+        for (uint32_t w = 0; w < kResidentWaves; ++w) dot += part[32 * w];
+        const uint32_t key = row < a.R ? ((uint32_t)(na + nb_row - 2 * dot) << 5) | var_row : 0xffffffffu;
+        const uint32_t best = wave_min_u32_dpp(key);
+        const uint32_t tag = a.tag0 + i;
+        unsigned long long *set = a.slots + (size_t)(i & 1) * 64 * kSlotStride;
+        if (tid == 0)
+            __hip_atomic_store(set + (size_t)n * kSlotStride, ((unsigned long long)tag << 32) | (best >> 5), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 3);
+
+        // (3) while the words travel: the next image's variants into LDS, the requests for the image after it, and the
+        // part of the update that does not need the best match (the neuron's own best variant is known)
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < SV; ++u) {
+                const uint32_t t = tid + kResidentThreads * u;
+                if (t < n_var) var_next[t] = sv[u];
+            }
+            for (uint32_t t = tid + kResidentThreads * SV; t < n_var; t += kResidentThreads) var_next[t] = rot[(size_t)(i + 1) * a.rot_stride + t];
+            load_fragments(pb + a.pb_stride, wave);
+            nb_row = (int)a.nb[(size_t)(i + 1) * a.nb_stride + row];
+            if (i + 2 < a.images) load_variants(rot + (size_t)(i + 2) * a.rot_stride);
+        }
+        const uint32_t dec = (uint32_t)__builtin_amdgcn_readlane((int)dec_lane, (int)(best & 31u));
+        const float *x = var_cur + (dec >> 8);
+        const uint32_t shift = dec & 0xffu;
+        float diff[EPT];
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) diff[u] = __fsub_rn(wv[u], x[(uint32_t)(sp[u] >> shift) & 0xffffu]);
+
+        // (4) the first wave waits for all words
+        if (wave == 0) {
+            unsigned long long v = 0;
+            uint32_t spins = 0;
+            bool all_in = false, gave_up = false;
+            while (!all_in && !gave_up) {
+                v = lane < N ? __hip_atomic_load(set + (size_t)lane * kSlotStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                             : (unsigned long long)tag << 32;
+                all_in = __all((uint32_t)(v >> 32) == tag) != 0;
+                if (!all_in)
+                    gave_up = __any(++spins > a.spin_limit || __hip_atomic_load(a.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) != 0;
+            }
+            if (gave_up) {
+                if (lane == 0) {
+                    __hip_atomic_store(a.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_bmu = 0xffffffffu;
+                }
+            } else {
+                // best match: first minimum of the distances (Trainer.h:164-168)
+                const uint32_t dist = lane < N ? (uint32_t)v : 0xffffffffu, lowest = wave_min_u32_dpp(dist);
+                const uint32_t bmu = (uint32_t)__builtin_ctzll(__ballot(dist == lowest));
+                if (lane == 0) s_bmu = bmu;
+            }
+        }
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 4);
+        __syncthreads();
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 5);
+        const uint32_t bmu = s_bmu;
+        if (bmu == 0xffffffffu) return;                   // somebody gave up: every block leaves, nothing is written back
+        const float f = s_f[bmu];
+        if (n == 0 && tid == 0) a.bmu_out[i] = bmu;
+
+        // (5) the rest of the update (Trainer.h:175), the neuron's operand row and its norm
+        if (f != 0.0f) {
+            int sq = 0;
+#pragma unroll
+            for (int u = 0; u < EPT; ++u) {
+                const float nv = __fsub_rn(wv[u], __fmul_rn(diff[u], f));
+                wv[u] = nv;
+                const int h = quantise(nv, 255.0f) - 128;
+                ((signed char *)s_op)[cb[u]] = (signed char)h;
+                sq += (h * h) & (int)in_region[u];
+            }
+            sq = wave_sum_i32_dpp(sq);
+            if (lane == 0) s_sq[wave] = sq;
+        }
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 6);
+        __syncthreads();
+        if (i + 2 == a.images) PROBE(kProbeResident, n, 7);
+        if (f != 0.0f) {
+            na = 0;
+#pragma unroll
+            for (uint32_t w = 0; w < kResidentWaves; ++w) na += s_sq[w];
+        }
+    }
+
+    // the group's result, into the other buffers
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        const uint32_t j = tid + kResidentThreads * u;
+        if (j < S) som_next[(size_t)n * S + j] = wv[u];
+    }
+    if (tid < 2 * KS)
+        *(v4i *)(Pa_next + ((((size_t)(n >> 5) * KS) * 64 + (n & 31)) << 4) + (size_t)(tid >> 1) * 1024 + (tid & 1) * 512) = s_op[tid];
+    if (tid == 0) a.na_next[n] = (long long)na;
+}
+
+// m_update_info[bmu]++ for the images of a group (Trainer.h:302-303), after a resident launch that went through.
+__global__ __launch_bounds__(256) void k_count_best_matches(const uint32_t *__restrict__ bmu, uint32_t images, uint32_t *__restrict__ counts)
+{
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < images) atomicAdd(&counts[bmu[t]], 1u);
+}
+
 // Decode keys: distance (optionally square-rooted for the mapper, Mapper.h:206), exact
 // integer sum, best rotation.  Integer modes: distance = float(double(ssd) / factor^2).
 __global__ __launch_bounds__(256) void k_finalize(const unsigned long long *__restrict__ key, float *__restrict__ dist,
@@ -1961,6 +2200,14 @@ struct pink_hip_ctx {
     v4i *d_gPa_alt = nullptr;             // small uint8 trainers: the SOM operand alternates between two buffers
     uint32_t pa_cur = 0;                   // ... which of them holds the current SOM
     bool small_train = false;              // ... one launch per image (k_train_small_u8)
+    // ... or one launch per group, the blocks exchanging a word per image (k_train_small_u8_resident): the group's
+    // result goes to the other buffers (d_som_alt, the other operand, the other norms) and becomes current when the
+    // launch reports that no block gave up waiting
+    bool resident_train = false;
+    float *d_som_alt = nullptr;
+    unsigned long long *d_slots = nullptr;
+    uint32_t *d_resident_error = nullptr, *h_resident_error = nullptr;
+    uint32_t exchange_tag = 1, spin_limit = 1u << 21;
     unsigned long long *d_src4 = nullptr;  // ... its per-element tables (see the kernel)
     uint32_t *d_kbyte = nullptr;
     uint32_t *d_grow = nullptr, *d_gvariant = nullptr;   // variant index -> row of the variant operand, and back
@@ -2525,6 +2772,64 @@ int run_train_small(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     return launch_check(ctx, "k_train_small_u8");
 }
 
+// The first `images` images of the current group in one resident launch (small uint8 trainers).  `went_through`
+// false: a block gave up waiting for the others (the device was not free to hold all blocks at once); nothing of
+// the context has changed then, the context stops using this form, and the caller trains the group image by image.
+int run_train_small_resident(pink_hip_ctx *ctx, uint32_t images, uint32_t *dev_bmu, bool *went_through)
+{
+    *went_through = false;
+    if (ctx->exchange_tag > 0xffffffffu - images) {        // the tags wrap: back to 1, over slots that hold none
+        HIP_TRY(ctx, hipMemsetAsync(ctx->d_slots, 0, kSlotWords * sizeof(unsigned long long), ctx->stream));
+        ctx->exchange_tag = 1;
+    }
+    ResidentTrain a{};
+    a.na_cur = ctx->d_gna + (size_t)ctx->na_cur * ctx->Np;
+    a.na_next = ctx->d_gna + (size_t)(ctx->na_cur ^ 1) * ctx->Np;
+    a.nb = ctx->d_gnb;
+    a.variant = ctx->d_gvariant;
+    a.bmu_out = dev_bmu;
+    a.slots = ctx->d_slots;
+    a.error = ctx->d_resident_error;
+    a.N = ctx->N; a.S = ctx->S; a.R = ctx->R; a.KS = ctx->gKS;
+    a.nstored = std::min(2 * std::max(ctx->nrr, 1u), ctx->R);
+    a.images = images; a.tag0 = ctx->exchange_tag; a.spin_limit = ctx->spin_limit;
+    a.rot_stride = ctx->R * ctx->S;
+    a.pb_stride = (ctx->Rp / 32) * ctx->gKS * 64;
+    a.nb_stride = ctx->Rp;
+    a.vp.D = ctx->D; a.vp.num_rot = ctx->cfg.num_rot; a.vp.nrr = std::max(ctx->nrr, 1u);
+    ctx->exchange_tag += images;
+    const v4i *pa = cur_gPa(ctx);
+    signed char *pa_next = (signed char *)(ctx->pa_cur ? ctx->d_gPa : ctx->d_gPa_alt);
+    const size_t lds = (size_t)2 * a.nstored * ctx->S * sizeof(float);
+    {
+        Timed t(ctx, kClsUpdate, images);
+#define LAUNCH_RESIDENT(...)                                                                                          \
+    hipLaunchKernelGGL((k_train_small_u8_resident<__VA_ARGS__>), dim3(ctx->N), dim3(kResidentThreads), lds, ctx->stream, ctx->d_som, \
+                       ctx->d_som_alt, ctx->d_rot, pa, pa_next, ctx->d_gPb, ctx->d_factors, ctx->d_src4, ctx->d_kbyte, a)
+        // (elements of a neuron per thread, k-steps per wave in one batch, variant elements per thread in registers)
+        const bool few_variant_elements = (size_t)a.nstored * ctx->S <= 4 * kResidentThreads;
+        if (ctx->S <= 1024 && few_variant_elements) LAUNCH_RESIDENT(2, 4, 4);
+        else if (ctx->S <= 1024) LAUNCH_RESIDENT(2, 4, 8);
+        else LAUNCH_RESIDENT(4, 8, 8);
+#undef LAUNCH_RESIDENT
+        TRY(launch_check(ctx, "k_train_small_u8_resident"));
+    }
+    HIP_TRY(ctx, hipMemcpyAsync(ctx->h_resident_error, ctx->d_resident_error, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (*ctx->h_resident_error) {
+        ctx->resident_train = false;
+        HIP_TRY(ctx, hipMemsetAsync(ctx->d_resident_error, 0, sizeof(uint32_t), ctx->stream));
+        return PINK_HIP_OK;
+    }
+    std::swap(ctx->d_som, ctx->d_som_alt);
+    ctx->pa_cur ^= 1;
+    ctx->na_cur ^= 1;
+    hipLaunchKernelGGL(k_count_best_matches, dim3((images + 255) / 256), dim3(256), 0, ctx->stream, dev_bmu, images, ctx->d_counts);
+    TRY(launch_check(ctx, "k_count_best_matches"));
+    *went_through = true;
+    return PINK_HIP_OK;
+}
+
 int run_finalize(pink_hip_ctx *ctx, uint32_t B, float *dev_dist, long long *dev_ssd, uint32_t *dev_best, bool do_sqrt)
 {
     Timed t(ctx, kClsFinal);
@@ -2544,10 +2849,11 @@ int free_all(pink_hip_ctx *ctx)
     void *bufs[] = {ctx->d_som, ctx->d_rot, ctx->d_cos, ctx->d_sin, ctx->d_factors, ctx->d_factors_t, ctx->d_region, ctx->d_key,
                     ctx->d_somP, ctx->d_somP_alt, ctx->d_bmu_group, ctx->d_rotT, ctx->d_bmu_scratch, ctx->d_dist, ctx->d_ssd, ctx->d_best,
                     ctx->d_Pa, ctx->d_Pb, ctx->d_na, ctx->d_nb, ctx->d_poff, ctx->d_need, ctx->d_inv,
-                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
+                    ctx->d_upos, ctx->d_aoff, ctx->d_kmask, ctx->d_gPa, ctx->d_gPa_alt, ctx->d_som_alt, ctx->d_slots, ctx->d_resident_error, ctx->d_src4, ctx->d_kbyte, ctx->d_gPb, ctx->d_gna, ctx->d_gnb, ctx->d_rtab, ctx->d_symoff, ctx->d_grow, ctx->d_gvariant, ctx->d_region4};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (void *p : {(void *)ctx->st_img, (void *)ctx->st_heat, (void *)ctx->st_best, (void *)ctx->st_bmu}) if (p) (void)hipFree(p);
     if (ctx->st_pin) (void)hipHostFree(ctx->st_pin);
+    if (ctx->h_resident_error) (void)hipHostFree(ctx->h_resident_error);
     for (int i = 0; i < 2; ++i) {
         if (ctx->pend_pin[i]) (void)hipHostFree(ctx->pend_pin[i]);
         if (ctx->pend_ev[i]) (void)hipEventDestroy(ctx->pend_ev[i]);
@@ -2861,6 +3167,10 @@ int init_ctx(pink_hip_ctx *ctx)
     if (ctx->trainer) {
         // images whose variants are prepared ahead of the sequential distance/update chain
         size_t b = c.max_batch ? c.max_batch : 64;
+        // small uint8 trainers (see k_train_small_u8_resident: one launch per group, the host waits for each): 256
+        if (!c.max_batch && ctx->gemm && ctx->pair_variants && c.kernel_choice == PINK_HIP_KERNEL_AUTO && c.ed_type == PINK_HIP_UINT8 &&
+            ctx->N <= 64 && ctx->R <= 32 && ctx->S <= 2048 && ctx->gKS <= 64)
+            b = 256;
         const size_t budget = (size_t)2 << 30;
         while (b > 1 && b * per_image > budget) b >>= 1;
         if (!c.max_batch) {
@@ -3036,6 +3346,25 @@ int init_ctx(pink_hip_ctx *ctx)
             // (limits are per kernel, not per context)
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8<8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 32768));
+            // resident over a launch group: every block needs a compute unit of its own for the whole launch
+            ctx->resident_train = ctx->N <= (uint32_t)ctx->num_cu;
+            if (const char *off = getenv("PINK_HIP_RESIDENT_TRAINER")) ctx->resident_train = ctx->resident_train && atoi(off) != 0;
+            if (ctx->resident_train) {
+                // (a test can make every wait give up at once, to see the group trained again image by image)
+                if (const char *limit = getenv("PINK_HIP_RESIDENT_SPIN_LIMIT")) ctx->spin_limit = (uint32_t)strtoul(limit, nullptr, 10);
+                TRY(dev_alloc(ctx, &ctx->d_som_alt, (size_t)ctx->N * ctx->S));
+                TRY(dev_alloc(ctx, &ctx->d_slots, (size_t)kSlotWords));
+                HIP_TRY(ctx, hipMemset(ctx->d_slots, 0, kSlotWords * sizeof(unsigned long long)));
+                TRY(dev_alloc(ctx, &ctx->d_resident_error, 1));
+                HIP_TRY(ctx, hipMemset(ctx->d_resident_error, 0, sizeof(uint32_t)));
+                if (hipHostMalloc((void **)&ctx->h_resident_error, sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
+                    ctx->h_resident_error = nullptr;
+                    return fail(ctx, PINK_HIP_ENOMEM, "pinned host allocation failed");
+                }
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8_resident<2, 4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8_resident<2, 4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)k_train_small_u8_resident<4, 8, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+            }
         }
         // one launch per image where the float32 distance kernel runs in its one-wave-per-SIMD form (see k_train_f32_dpp;
         // up to 256 neurons: measured with 512 allowed, 17 x 17 and 18 x 18 neurons at 720 variants train no faster this
@@ -3046,7 +3375,7 @@ int init_ctx(pink_hip_ctx *ctx)
         ctx->rows_f32_train = !ctx->fused_f32_train && c.ed_type == PINK_HIP_FLOAT && !ctx->f32gemm && ctx->d_somP && ctx->d_inv &&
                               B <= kReplayMax;
         if (ctx->fused_f32_train) TRY(dev_alloc(ctx, (uint32_t **)&ctx->d_somP_alt, (size_t)ctx->N * ctx->Epad + kDistOverrun));
-        if (ctx->fused_f32_train || ctx->rows_f32_train) TRY(dev_alloc(ctx, &ctx->d_bmu_group, B));
+        if (ctx->fused_f32_train || ctx->rows_f32_train || ctx->resident_train) TRY(dev_alloc(ctx, &ctx->d_bmu_group, B));
         TRY(dev_alloc(ctx, &ctx->d_factors, (size_t)ctx->N * ctx->N));
         HIP_TRY(ctx, hipMemcpy(ctx->d_factors, c.update_factors, (size_t)ctx->N * ctx->N * sizeof(float),
                                hipMemcpyHostToDevice));
@@ -3306,6 +3635,11 @@ int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n
             }
             TRY(run_update_replay(ctx, B, bmu));
             continue;
+        }
+        if (ctx->resident_train) {
+            bool went_through = false;
+            TRY(run_train_small_resident(ctx, B, dev_bmu_out ? dev_bmu_out + done : ctx->d_bmu_group, &went_through));
+            if (went_through) continue;
         }
         for (uint32_t b = 0; b < B; ++b) {
             if (ctx->small_train) {

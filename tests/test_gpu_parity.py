@@ -495,6 +495,49 @@ def test_train_over_shapes(N, C_, I, D, nrot, flip, ed, shape_, ed_type, n):
     assert np.array_equal(bits(d1), bits(d2)) and np.array_equal(ssd1, ssd2) and np.array_equal(best1, best2)
 
 
+SMALL_UINT8_SHAPES = [s for s in FUSED_TRAIN_SHAPES if s[8] == capi.UINT8 and s[0] <= 64 and s[4] * (2 if s[5] else 1) <= 32
+                      and s[1] * s[3] * s[3] <= 2048] + [
+    (64, 1, 28, 28, 4, True, 28, capi.QUADRATIC, capi.UINT8, 40),     # the 8 x 8 MNIST-sized trainer of the benchmark set
+    (1, 1, 16, 16, 4, True, 12, capi.QUADRATIC, capi.UINT8, 9),       # one neuron: an exchange with itself
+    (64, 1, 45, 45, 4, False, 45, capi.QUADRATIC, capi.UINT8, 6),     # 2025 elements: four per thread, 64 k-steps
+]
+
+
+@pytest.mark.parametrize("form", ["resident", "gives up", "off"])
+@pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_,ed_type,n", SMALL_UINT8_SHAPES)
+def test_small_uint8_trainer_forms(monkeypatch, N, C_, I, D, nrot, flip, ed, shape_, ed_type, n, form):
+    """Small uint8 trainers run a whole launch group in one resident launch whose blocks exchange a word per image;
+    when a block gives up waiting for the others (forced here by a wait limit of zero polls: every kernel still
+    ends by itself) nothing of the context has changed and the group is trained again with one launch per image,
+    as it is with the resident form switched off.  All three against the oracle, bit for bit."""
+    say("small uint8 trainer", form, N, C_, I, D, nrot, flip, ed, shape_, n)
+    if form == "gives up":
+        monkeypatch.setenv("PINK_HIP_RESIDENT_SPIN_LIMIT", "0")
+    if form == "off":
+        monkeypatch.setenv("PINK_HIP_RESIDENT_TRAINER", "0")
+    rng = np.random.default_rng(N * 7 + I + nrot)
+    som0 = rng.random((N, C_ * D * D), dtype=np.float32)
+    imgs = rng.random((n, C_, I, I), dtype=np.float32)
+    F = capi.make_update_factors(capi.CARTESIAN, [N], capi.GAUSSIAN, 1.0, 0.5)
+    F[F < 0.01] = 0.0
+    s = O.shape(N, C_, I, D, nrot, flip, ed, shape_, ed_type)
+    want = som0.copy()
+    obmu = O.train(s, want, imgs, F)
+    for max_batch in (0, 3):                                 # the whole call in one group; groups of three images
+        with capi.Context(N, C_, I, D, nrot, flip, ed, shape_, ed_type, F, max_batch=max_batch) as ctx:
+            ctx.set_som(som0)
+            bmu = np.concatenate([ctx.train(imgs[:2]), ctx.train(imgs[2:])])
+            som = ctx.get_som()
+            counts = ctx.update_counts()
+            d1, ssd1, best1 = ctx.distance(imgs[0])          # the operand and norms the trainer left behind
+            ctx.set_som(som)
+            d2, ssd2, best2 = ctx.distance(imgs[0])
+        assert np.array_equal(bmu, obmu), max_batch
+        assert np.array_equal(bits(som), bits(want)), max_batch
+        assert np.array_equal(counts, np.bincount(obmu, minlength=N)), max_batch
+        assert np.array_equal(bits(d1), bits(d2)) and np.array_equal(ssd1, ssd2) and np.array_equal(best1, best2)
+
+
 @pytest.mark.parametrize("N,ed_type", [(9, capi.FLOAT), (9, capi.UINT8), (530, capi.UINT8)])
 def test_train_with_any_factor_matrix(N, ed_type):
     # the C interface takes any N x N matrix, not only the symmetric ones that a distance functor gives
@@ -699,7 +742,7 @@ def test_mfma_kernel_refused_where_it_does_not_apply():
     # launch for the neurons' full images and the last image's update
     ("cfg0", capi.KERNEL_AUTO, 5, 2),
     ("cfg4", capi.KERNEL_MFMA_GEMM, 5, 5),
-    ("cfg4", capi.KERNEL_AUTO, 0, 5),       # a small uint8 trainer: distance, best match and update in one launch per image
+    ("cfg4", capi.KERNEL_AUTO, 0, 5),       # a small uint8 trainer: one resident launch per group, counted once per image
 ])
 def test_profiling_counts_launches(name, choice, distance_launches, update_launches):
     w = synthetic.WORKLOADS[name]
