@@ -1780,13 +1780,15 @@ __global__ __launch_bounds__(256) void k_train_small_u8(float *__restrict__ som,
 // else crosses between blocks, so no fences: the payload rides in the atomic word.  Two sets of slots take turns
 // (a block can be at most one image ahead of another).  The exchange costs about 1.4 us, where a launch boundary
 // with the distance matrix worked out again in every block costs 5.
-// Every wait is bounded: a wave that does not see all words within `spin_limit` polls raises `error`, polling
-// waves leave when they see it raised, a block that leaves stops publishing, so every block leaves.  The group's
+// Every wait is bounded: a wave that does not see all words within `spin_limit` polls raises `error` and marks its
+// block's slots, polling waves leave when they see such a mark, a block that leaves stops publishing, so every
+// block leaves.  The group's
 // results go to the OTHER buffers (weights, operand, norms); the host looks at `error` after the launch and only
 // then makes them the current ones, or trains the group again, image by image, from the untouched current ones.
 // ---------------------------------------------------------------------------------
 constexpr uint32_t kSlotStride = 16;                      // 64-bit words between two blocks' slots (128 bytes)
 constexpr uint32_t kSlotWords = 2 * 64 * kSlotStride;     // two sets of 64 slots
+constexpr uint32_t kGaveUpTag = 0xffffffffu;              // in a slot: its block has left the launch
 
 struct ResidentTrain {
     const long long *na_cur;
@@ -1941,14 +1943,17 @@ __global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__
             unsigned long long v = 0;
             uint32_t spins = 0;
             bool all_in = false, gave_up = false;
+            // (one load per poll: a block that gives up says so in its own slots, with a tag no image has)
             while (!all_in && !gave_up) {
                 v = lane < N ? __hip_atomic_load(set + (size_t)lane * kSlotStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                              : (unsigned long long)tag << 32;
                 all_in = __all((uint32_t)(v >> 32) == tag) != 0;
-                if (!all_in)
-                    gave_up = __any(++spins > a.spin_limit || __hip_atomic_load(a.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) != 0;
+                if (!all_in) gave_up = __any(++spins > a.spin_limit || (uint32_t)(v >> 32) == kGaveUpTag) != 0;
             }
             if (gave_up) {
+                if (lane < 2)
+                    __hip_atomic_store(a.slots + ((size_t)lane * 64 + n) * kSlotStride, (unsigned long long)kGaveUpTag << 32, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
                 if (lane == 0) {
                     __hip_atomic_store(a.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     s_bmu = 0xffffffffu;
@@ -2778,7 +2783,7 @@ int run_train_small(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
 int run_train_small_resident(pink_hip_ctx *ctx, uint32_t images, uint32_t *dev_bmu, bool *went_through)
 {
     *went_through = false;
-    if (ctx->exchange_tag > 0xffffffffu - images) {        // the tags wrap: back to 1, over slots that hold none
+    if (ctx->exchange_tag > 0xfffffff0u - images) {        // the tags wrap: back to 1, over slots that hold none
         HIP_TRY(ctx, hipMemsetAsync(ctx->d_slots, 0, kSlotWords * sizeof(unsigned long long), ctx->stream));
         ctx->exchange_tag = 1;
     }
@@ -2819,6 +2824,7 @@ int run_train_small_resident(pink_hip_ctx *ctx, uint32_t images, uint32_t *dev_b
     if (*ctx->h_resident_error) {
         ctx->resident_train = false;
         HIP_TRY(ctx, hipMemsetAsync(ctx->d_resident_error, 0, sizeof(uint32_t), ctx->stream));
+        HIP_TRY(ctx, hipMemsetAsync(ctx->d_slots, 0, kSlotWords * sizeof(unsigned long long), ctx->stream));
         return PINK_HIP_OK;
     }
     std::swap(ctx->d_som, ctx->d_som_alt);
