@@ -56,7 +56,7 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg3", "distance"): (247.797e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
     ("cfg3", "update"): (73.892e6 + 47.153e6 + (295.051e6 + 94.661e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg4", "update"): (1.231e6 + 0.303e6, "profiles/cfg4_train_u8_counters.txt"),     # the one launch per image
+    ("cfg4", "update"): ((85.610e6 + 0.835e6) / 256, "profiles/cfg4_train_u8_counters.txt"),     # the resident launch of 256 images
 }
 
 # Images per step of the workloads that ride along in `all_configs` (the headline workload always
@@ -110,7 +110,8 @@ def distance_path_name(w, path, times):
             return "float32 vector ALU, one (neuron, variant) pair per lane, DPP broadcast; the launch also applies the update of the image before"
         return "float32 vector ALU, one (neuron, variant) pair per lane"
     if w.mode == "train" and path == capi.KERNEL_MFMA_GEMM and times["distance"][0] == 0:
-        return "int8 MFMA inside the one launch per image of a small uint8 trainer (distances, best match, update)"
+        return ("int8 MFMA inside the resident launch of a small uint8 trainer (one launch per group of images: distances, "
+                "best match, update; one block per neuron, a 64-bit word per block and image exchanged through memory)")
     return {capi.KERNEL_VALU: "integer vector ALU", capi.KERNEL_MFMA: "int8 MFMA, image-side symmetries, SOM operand in LDS",
             capi.KERNEL_MFMA_SYM: "int8 MFMA, SOM-side symmetries, SOM operand in registers",
             capi.KERNEL_MFMA_GEMM: "int8 MFMA GEMM, one launch, 64x64 or 32x32 tiles over the whole k range, finished by their blocks",
@@ -302,8 +303,10 @@ def run_workload(name, steps, warmup, n_images, kernel, cpu_budget_s, host_inclu
             notes = ("vector-ALU bound (exact bilinear arithmetic per operand byte), far from HBM: "
                      "algorithmic bytes = image read + packed operand written")
         if dominant == "update" and times["distance"][0] == 0:
-            notes = ("a small uint8 trainer: distances, best match and update of an image in one launch (class 'update'); "
-                     "bound by the launch's fixed cost and one memory round trip, not by HBM: no roofline claimed")
+            notes = ("a small uint8 trainer: distances, best match and update of a whole group of images in one resident "
+                     "launch (class 'update'), one block per neuron; per image the blocks exchange one 64-bit word each "
+                     "through memory (store, then polls: about 0.9 us) around about 1 us of lone-wave instruction issue; "
+                     "bound by that chain, not by HBM: no roofline claimed")
     traffic = COUNTER_TRAFFIC_PER_IMAGE.get((name, dominant))
     roofline = {
         "kernel": dominant, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,

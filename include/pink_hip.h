@@ -135,7 +135,7 @@ int pink_hip_get_som(pink_hip_ctx *ctx, float *host_som);
  * m_update_info (Trainer.h:302-303); the call then returns when they are there.
  * With bmu_out NULL and up to 128 KiB of images the call only copies the images into a
  * pinned buffer and returns (operator() returns nothing either); they are trained, in
- * order, a launch group (up to 64 images) at a time: when the group is full or when any
+ * order, a launch group (up to 64 images; 256 for small uint8 trainers) at a time: when the group is full or when any
  * other call on the context follows.  A loop of per-image calls then runs at the rate of
  * the kernels (the rotation of a group is one launch), not of per-image launches and
  * round trips, and leaves the weights of training call by call.  pink_hip_get_som,
@@ -146,7 +146,15 @@ int pink_hip_train(pink_hip_ctx *ctx, const float *host_images, uint32_t n_image
  * best match, over all images this context has trained, counted on the device. */
 int pink_hip_update_counts(pink_hip_ctx *ctx, uint32_t *host_counts_out);
 /* Same with the images already on the device and the BMUs left on the device;
- * asynchronous on the context's stream (see pink_hip_synchronize). */
+ * asynchronous on the context's stream (see pink_hip_synchronize).  A small uint8 trainer
+ * (at most 64 neurons, 32 variants, 2048 elements per neuron) trains a launch group of up
+ * to 256 images in ONE launch whose blocks stay on the device and exchange one word per
+ * image; the host waits for each such launch and learns from it whether every block saw
+ * the others in time (they do unless other work keeps the device's compute units busy for
+ * seconds).  If not, nothing of the context has changed, the group is trained again with
+ * one launch per image, and the context stays with that form.  The environment variable
+ * PINK_HIP_RESIDENT_TRAINER=0, read when a context is created, selects the one launch per
+ * image from the start. */
 int pink_hip_train_device(pink_hip_ctx *ctx, const float *dev_images, uint32_t n_images, uint32_t *dev_bmu_out);
 
 /* Mapper<...,true>::operator()(Data const&) (Mapper.h:181-208) for n_images images:

@@ -2807,7 +2807,7 @@ int run_train_small_resident(pink_hip_ctx *ctx, uint32_t images, uint32_t *dev_b
     signed char *pa_next = (signed char *)(ctx->pa_cur ? ctx->d_gPa : ctx->d_gPa_alt);
     const size_t lds = (size_t)2 * a.nstored * ctx->S * sizeof(float);
     {
-        Timed t(ctx, kClsUpdate, images);
+        Timed t(ctx, kClsUpdate);
 #define LAUNCH_RESIDENT(...)                                                                                          \
     hipLaunchKernelGGL((k_train_small_u8_resident<__VA_ARGS__>), dim3(ctx->N), dim3(kResidentThreads), lds, ctx->stream, ctx->d_som, \
                        ctx->d_som_alt, ctx->d_rot, pa, pa_next, ctx->d_gPb, ctx->d_factors, ctx->d_src4, ctx->d_kbyte, a)

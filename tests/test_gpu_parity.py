@@ -742,7 +742,7 @@ def test_mfma_kernel_refused_where_it_does_not_apply():
     # launch for the neurons' full images and the last image's update
     ("cfg0", capi.KERNEL_AUTO, 5, 2),
     ("cfg4", capi.KERNEL_MFMA_GEMM, 5, 5),
-    ("cfg4", capi.KERNEL_AUTO, 0, 5),       # a small uint8 trainer: one resident launch per group, counted once per image
+    ("cfg4", capi.KERNEL_AUTO, 0, 1),       # a small uint8 trainer: one resident launch for the group
 ])
 def test_profiling_counts_launches(name, choice, distance_launches, update_launches):
     w = synthetic.WORKLOADS[name]
