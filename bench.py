@@ -56,7 +56,7 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg3", "distance"): (247.797e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
     ("cfg3", "update"): (73.892e6 + 47.153e6 + (295.051e6 + 94.661e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
-    ("cfg4", "update"): ((85.610e6 + 0.835e6) / 256, "profiles/cfg4_train_u8_counters.txt"),     # the resident launch of 256 images
+    ("cfg4", "update"): ((85.604e6 + 0.835e6) / 256, "profiles/cfg4_train_u8_counters.txt"),     # the resident launch of 256 images
 }
 
 # Images per step of the workloads that ride along in `all_configs` (the headline workload always

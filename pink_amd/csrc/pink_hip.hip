@@ -1817,9 +1817,9 @@ __global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__
     extern __shared__ float s_var[];                      // the stored variants of this image and of the next one
     __shared__ v4i s_op[128 + 1];                         // this neuron's operand row: [k-step][half of the k-step]; one spare
     __shared__ v4i s_part[kResidentWaves][2][4];          // [wave][half][16 accumulators]
-    __shared__ float s_f[64];
     __shared__ int s_sq[kResidentWaves];
-    __shared__ uint32_t s_bmu;
+    __shared__ uint2 s_bmu_f;                             // the best match (all ones: leave) and this neuron's factor for it
+    uint32_t &s_bmu = s_bmu_f.x;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = blockIdx.x;
     const uint32_t N = a.N, S = a.S, KS = a.KS, n_var = a.nstored * S;
     // (a launch that follows one that gave up leaves at once; one thread looks, so the whole block decides alike)
@@ -1842,7 +1842,7 @@ __global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__
         cb[u] = kb == 0xffffffffu ? 128u * 16u + (tid & 15u) : ((kb >> 9) << 4) | (kb & 15u);
         sp[u] = src4[j];
     }
-    if (tid < 64) s_f[tid] = tid < N ? factors[(size_t)tid * N + n] : 0.0f;
+    const float f_if = lane < N ? factors[(size_t)lane * N + n] : 0.0f;     // the factor, should neuron `lane` be the best match
     // (k-steps past the end hold zeros: a wave whose share of the k-steps ends early multiplies by them)
     if (tid < 128) {
         const v4i zero = {0, 0, 0, 0};
@@ -1886,14 +1886,17 @@ __global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__
 
         // (1) this neuron against all variants: this wave's k-steps (the operand row out of LDS first: a lone
         // wave waits out every LDS read it issues between two MFMAs)
+        // (the first batch whatever KS: a wave with no k-step of its own multiplies by the zero k-steps)
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        for (uint32_t first = wave; first < KS; first += kResidentWaves * KSW) {
-            if (first != wave) load_fragments(pb, first);
+        for (uint32_t first = wave;;) {
             v4i fa[KSW];
 #pragma unroll
             for (int u = 0; u < KSW; ++u) fa[u] = s_op[min(first + kResidentWaves * u, 63u) * 2 + (lane >> 5)];
 #pragma unroll
             for (int u = 0; u < KSW; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[u], fa[u], acc, 0, 0, 0);
+            first += kResidentWaves * KSW;
+            if (first >= KS) break;
+            load_fragments(pb, first);
         }
         if (i + 2 == a.images) PROBE(kProbeResident, n, 1);
         if ((lane & 31) == 0) {
@@ -1956,21 +1959,23 @@ __global__ __launch_bounds__(512) void k_train_small_u8_resident(const float *__
                                        __HIP_MEMORY_SCOPE_AGENT);
                 if (lane == 0) {
                     __hip_atomic_store(a.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    s_bmu = 0xffffffffu;
+                    s_bmu_f = make_uint2(0xffffffffu, 0u);
                 }
             } else {
                 // best match: first minimum of the distances (Trainer.h:164-168)
                 const uint32_t dist = lane < N ? (uint32_t)v : 0xffffffffu, lowest = wave_min_u32_dpp(dist);
                 const uint32_t bmu = (uint32_t)__builtin_ctzll(__ballot(dist == lowest));
-                if (lane == 0) s_bmu = bmu;
+                const uint32_t f_bits = (uint32_t)__builtin_amdgcn_readlane(__builtin_bit_cast(int, f_if), (int)bmu);
+                if (lane == 0) s_bmu_f = make_uint2(bmu, f_bits);
             }
         }
         if (i + 2 == a.images) PROBE(kProbeResident, n, 4);
         __syncthreads();
         if (i + 2 == a.images) PROBE(kProbeResident, n, 5);
-        const uint32_t bmu = s_bmu;
+        const uint2 bmu_f = s_bmu_f;
+        const uint32_t bmu = bmu_f.x;
         if (bmu == 0xffffffffu) return;                   // somebody gave up: every block leaves, nothing is written back
-        const float f = s_f[bmu];
+        const float f = __builtin_bit_cast(float, bmu_f.y);
         if (n == 0 && tid == 0) a.bmu_out[i] = bmu;
 
         // (5) the rest of the update (Trainer.h:175), the neuron's operand row and its norm
