@@ -3363,6 +3363,8 @@ int init_ctx(pink_hip_ctx *ctx)
             if (ctx->resident_train) {
                 // (a test can make every wait give up at once, to see the group trained again image by image)
                 if (const char *limit = getenv("PINK_HIP_RESIDENT_SPIN_LIMIT")) ctx->spin_limit = (uint32_t)strtoul(limit, nullptr, 10);
+                // (... or start the tags of the exchange just below the value where they wrap, which 2^32 images take)
+                if (const char *tag = getenv("PINK_HIP_RESIDENT_FIRST_TAG")) ctx->exchange_tag = std::max(1u, (uint32_t)strtoul(tag, nullptr, 10));
                 TRY(dev_alloc(ctx, &ctx->d_som_alt, (size_t)ctx->N * ctx->S));
                 TRY(dev_alloc(ctx, &ctx->d_slots, (size_t)kSlotWords));
                 HIP_TRY(ctx, hipMemset(ctx->d_slots, 0, kSlotWords * sizeof(unsigned long long)));

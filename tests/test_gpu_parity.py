@@ -503,18 +503,21 @@ SMALL_UINT8_SHAPES = [s for s in FUSED_TRAIN_SHAPES if s[8] == capi.UINT8 and s[
 ]
 
 
-@pytest.mark.parametrize("form", ["resident", "gives up", "off"])
+@pytest.mark.parametrize("form", ["resident", "gives up", "off", "tags wrap"])
 @pytest.mark.parametrize("N,C_,I,D,nrot,flip,ed,shape_,ed_type,n", SMALL_UINT8_SHAPES)
 def test_small_uint8_trainer_forms(monkeypatch, N, C_, I, D, nrot, flip, ed, shape_, ed_type, n, form):
     """Small uint8 trainers run a whole launch group in one resident launch whose blocks exchange a word per image;
     when a block gives up waiting for the others (forced here by a wait limit of zero polls: every kernel still
     ends by itself) nothing of the context has changed and the group is trained again with one launch per image,
-    as it is with the resident form switched off.  All three against the oracle, bit for bit."""
+    as it is with the resident form switched off.  All against the oracle, bit for bit."""
     say("small uint8 trainer", form, N, C_, I, D, nrot, flip, ed, shape_, n)
     if form == "gives up":
         monkeypatch.setenv("PINK_HIP_RESIDENT_SPIN_LIMIT", "0")
     if form == "off":
         monkeypatch.setenv("PINK_HIP_RESIDENT_TRAINER", "0")
+    if form == "tags wrap":
+        # the exchange tags every image with a running 32-bit number; start it where the second call passes the end
+        monkeypatch.setenv("PINK_HIP_RESIDENT_FIRST_TAG", str(0xfffffff0 - n + 1))
     rng = np.random.default_rng(N * 7 + I + nrot)
     som0 = rng.random((N, C_ * D * D), dtype=np.float32)
     imgs = rng.random((n, C_, I, I), dtype=np.float32)
