@@ -1298,8 +1298,18 @@ __global__ __launch_bounds__(256) void k_update(float *__restrict__ som, const f
     __shared__ uint32_t s_idx[256];
     __shared__ float s_fcol[kFactorColumnMax];
     const uint32_t tid = threadIdx.x;
-    const uint32_t n = blockIdx.y, part = blockIdx.x;
-    const uint32_t probe_block = blockIdx.y * gridDim.x + blockIdx.x;
+    // Block (part, n); or, where the update also refreshes the byte planes of the integer GEMM's operand, the blocks of
+    // the four neurons whose 16-byte pieces share a 64-byte line of the planes on ONE XCD (workgroups go to the XCDs
+    // round-robin by linear id): its L2 then merges the four neurons' pieces into whole lines, where four L2s would
+    // each write the line back in parts.  The grid's x then counts (XCD, neuron in the four, group of eight fours).
+    uint32_t n = blockIdx.y, part = blockIdx.x;
+    if (up.Pa) {
+        const uint32_t x = blockIdx.x, four = (x >> 5) * 8 + (x & 7);
+        n = four * 4 + ((x >> 3) & 3);
+        part = blockIdx.y;
+        if (n >= N) return;
+    }
+    const uint32_t probe_block = n * parts + part;
     PROBE(kProbeUpdate, probe_block, 0);
     // The factor of this neuron depends on the best match, the neuron's column of the factor matrix does not: it is
     // requested with the keys (factors_t is the matrix transposed, so the column is contiguous) and waits in LDS.
@@ -2665,8 +2675,10 @@ int run_update(pink_hip_ctx *ctx, uint32_t slot, uint32_t *dev_bmu_out)
     }
     VariantPair vp{};
     if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
+    // (see the kernel: with the byte planes, the four neurons that share lines of them on one XCD)
+    const dim3 grid = up.Pa ? dim3(32 * ((ctx->N + 31) / 32), parts) : dim3(parts, ctx->N);
 #define LAUNCH_UPDATE(U_)                                                                                        \
-    hipLaunchKernelGGL(k_update<U_>, dim3(parts, ctx->N), dim3(256), 0, ctx->stream, ctx->d_som,                   \
+    hipLaunchKernelGGL(k_update<U_>, grid, dim3(256), 0, ctx->stream, ctx->d_som,                                  \
                        ctx->d_rot + (size_t)slot * ctx->R * ctx->S, ctx->d_key + (size_t)slot * ctx->N, ctx->d_factors_t, \
                        dev_bmu_out, ctx->N, ctx->S, parts, ctx->shift, ctx->d_somP,                                \
                        ctx->fused_som ? ctx->d_kbyte : ctx->gemm ? nullptr : ctx->d_inv, ctx->Epad,                \
