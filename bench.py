@@ -53,9 +53,9 @@ COUNTER_TRAFFIC_PER_IMAGE = {
     ("cfg1", "distance"): ((214.632e6 + 1.639e6) / 2048, "profiles/cfg1_map_u8_counters.txt"),
     ("cfg2", "distance"): (32.971e6 + 0.069e6, "profiles/cfg2_train_u16_counters.txt"),
     ("cfg2", "update"): (28.845e6 + 17.831e6, "profiles/cfg2_train_u16_counters.txt"),
-    ("cfg3", "distance"): (247.797e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "distance"): (252.417e6 + 0.576e6, "profiles/cfg3_train_f32_3ch_counters.txt"),
     # the operand rows per image and a sixteenth of the launch that brings the neurons' full images up to date
-    ("cfg3", "update"): (73.892e6 + 47.153e6 + (295.051e6 + 94.661e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
+    ("cfg3", "update"): (73.894e6 + 47.153e6 + (323.973e6 + 95.049e6) / 16, "profiles/cfg3_train_f32_3ch_counters.txt"),
     ("cfg4", "update"): ((85.604e6 + 0.835e6) / 256, "profiles/cfg4_train_u8_counters.txt"),     # the resident launch of 256 images
 }
 

@@ -1549,6 +1549,7 @@ __global__ __launch_bounds__(256) void k_update_rows(float *__restrict__ somP, c
 // all images side by side first (one thread each) and kept in LDS, so the loop over the images is one
 // variant element and three operations per image with nothing that depends on the image before.
 constexpr uint32_t kReplayMax = 256;         // images per launch
+template <int EPT>       // elements per thread, 256 apart
 __global__ __launch_bounds__(256) void k_update_replay(float *__restrict__ som, const float *__restrict__ rot,
                                                        const unsigned long long *__restrict__ key, const float *__restrict__ factors,
                                                        const uint32_t *__restrict__ bmu, uint32_t images, uint32_t N, uint32_t S,
@@ -1558,7 +1559,9 @@ __global__ __launch_bounds__(256) void k_update_replay(float *__restrict__ som, 
     __shared__ uint32_t s_row[kReplayMax];   // stored row of the group's variants * 4 + how it is read
     // (neurons vary fastest over the grid: the blocks that run side by side then read the same stretch of elements of
     // whatever variants their neurons were closest to -- a few MB that stay in L2 -- and not whole variants)
-    const uint32_t n = blockIdx.x, j = blockIdx.y * 256 + threadIdx.x;
+    // (several elements per thread: what an image costs the thread beside its elements -- its row, how it is read, its
+    // factor, out of LDS -- is paid once for all of them)
+    const uint32_t n = blockIdx.x, j = blockIdx.y * (256 * EPT) + threadIdx.x;
     if (threadIdx.x < images) {
         const uint32_t i = threadIdx.x;
         const uint32_t r = (uint32_t)(key[(size_t)i * N + n] & ((1ull << shift) - 1ull));
@@ -1575,29 +1578,46 @@ __global__ __launch_bounds__(256) void k_update_replay(float *__restrict__ som, 
     }
     __syncthreads();
     if (j >= S) return;
-    // where element j sits in a stored variant read as it is, with columns, rows or both reversed (see k_update)
-    uint32_t src[4] = {j, j, j, j};
-    if (vp.D) {
-        const uint32_t D = vp.D, p = j % (D * D), x = p / D, y = p % D;
-        src[1] = j - p + x * D + (D - 1 - y);
-        src[2] = j - p + (D - 1 - x) * D + y;
-        src[3] = j - p + (D - 1 - x) * D + (D - 1 - y);
+    uint32_t jj[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) jj[e] = min(j + 256 * e, S - 1);      // (past the end: the last element again, not stored)
+    // where an element sits in a stored variant read as it is, with columns, rows or both reversed (see k_update)
+    uint32_t src[EPT][4];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        src[e][0] = src[e][1] = src[e][2] = src[e][3] = jj[e];
+        if (vp.D) {
+            const uint32_t D = vp.D, p = jj[e] % (D * D), x = p / D, y = p % D;
+            src[e][1] = jj[e] - p + x * D + (D - 1 - y);
+            src[e][2] = jj[e] - p + (D - 1 - x) * D + y;
+            src[e][3] = jj[e] - p + (D - 1 - x) * D + (D - 1 - y);
+        }
     }
-    float w = som[(size_t)n * S + j];
+    float w[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) w[e] = som[(size_t)n * S + jj[e]];
     for (uint32_t i0 = 0; i0 < images; i0 += 8) {
-        float x[8], f[8];
+        float x[8][EPT], f[8];
 #pragma unroll
         for (uint32_t u = 0; u < 8; ++u) {
             const uint32_t i = min(i0 + u, images - 1);
             const uint32_t rw = s_row[i], which = rw & 3;
             f[u] = i0 + u < images ? s_f[i] : 0.0f;
-            x[u] = rot[(size_t)(rw >> 2) * S + (which == 0 ? src[0] : which == 1 ? src[1] : which == 2 ? src[2] : src[3])];
+            const float *row = rot + (size_t)(rw >> 2) * S;
+#pragma unroll
+            for (int e = 0; e < EPT; ++e)
+                x[u][e] = row[which == 0 ? src[e][0] : which == 1 ? src[e][1] : which == 2 ? src[e][2] : src[e][3]];
         }
 #pragma unroll
         for (uint32_t u = 0; u < 8; ++u)
-            if (f[u] != 0.0f) w = __fsub_rn(w, __fmul_rn(__fsub_rn(w, x[u]), f[u]));
+            if (f[u] != 0.0f) {
+#pragma unroll
+                for (int e = 0; e < EPT; ++e) w[e] = __fsub_rn(w[e], __fmul_rn(__fsub_rn(w[e], x[u][e]), f[u]));
+            }
     }
-    som[(size_t)n * S + j] = w;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e)
+        if (j + 256 * e < S) som[(size_t)n * S + j + 256 * e] = w[e];
 }
 
 // ---------------------------------------------------------------------------------
@@ -2757,9 +2777,17 @@ int run_update_replay(pink_hip_ctx *ctx, uint32_t images, const uint32_t *dev_bm
     if (ctx->pair_variants) { vp.D = ctx->D; vp.num_rot = ctx->cfg.num_rot; vp.nrr = std::max(ctx->nrr, 1u); }
     for (uint32_t first = 0; first < images; first += kReplayMax) {
         const uint32_t count = std::min(kReplayMax, images - first);
-        hipLaunchKernelGGL(k_update_replay, dim3(ctx->N, (ctx->S + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_som,
-                           ctx->d_rot + (size_t)first * ctx->R * ctx->S, ctx->d_key + (size_t)first * ctx->N, ctx->d_factors,
-                           dev_bmu + first, count, ctx->N, ctx->S, ctx->R, ctx->shift, vp);
+#define LAUNCH_REPLAY(EPT_)                                                                                                   \
+    hipLaunchKernelGGL(k_update_replay<EPT_>, dim3(ctx->N, (ctx->S + 256 * EPT_ - 1) / (256 * EPT_)), dim3(256), 0, ctx->stream, \
+                       ctx->d_som, ctx->d_rot + (size_t)first * ctx->R * ctx->S, ctx->d_key + (size_t)first * ctx->N,            \
+                       ctx->d_factors, dev_bmu + first, count, ctx->N, ctx->S, ctx->R, ctx->shift, vp)
+        // (large SOMs: several elements per thread -- 1600 neurons of 3 x 70 x 70: 13.6 us per image with one, 10.2 with
+        // two, 9.0 with four; small ones need the blocks -- 100 neurons of 45 x 45: 0.42, 0.46)
+        const size_t weights = (size_t)ctx->N * ctx->S;
+        if (weights >= ((size_t)1 << 22)) LAUNCH_REPLAY(4);
+        else if (weights >= ((size_t)1 << 20)) LAUNCH_REPLAY(2);
+        else LAUNCH_REPLAY(1);
+#undef LAUNCH_REPLAY
         TRY(launch_check(ctx, "k_update_replay"));
     }
     return PINK_HIP_OK;
